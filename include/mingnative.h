@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MN_VERSION 124 /* 0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
+#define MN_VERSION 125 /* 0.1.25: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
                           mn_llm and mn_llm_tp (zero = bf16: callers of 0.1.10 that zero-fill the structs are unchanged),
                           mn_quant_fp8_rows / mn_dequant_fp8_rows / mn_stream_mfma_w8 / mn_stream_mfma_grouped_w8 */
 
@@ -58,7 +58,7 @@ MN_API int mn_num_cus(void);
  * mn_struct_layout(which, offsets, cap) writes offsetof(every field, in declaration order) into offsets[0 .. min(n, cap)) and
  * returns the field count n (MN_EINVAL for an unknown `which`). */
 enum mn_struct_id { MN_STRUCT_SKINNY_ARGS = 0, MN_STRUCT_RF_HEAD = 1, MN_STRUCT_LLM = 2, MN_STRUCT_SEMDEC = 3, MN_STRUCT_TP_COMM = 4,
-                    MN_STRUCT_LLM_TP = 5 };
+                    MN_STRUCT_LLM_TP = 5, MN_STRUCT_SEQ_LAYER = 6, MN_STRUCT_SEQ_MODEL = 7, MN_STRUCT_SEQ_STATE = 8 };
 MN_API size_t mn_sizeof_skinny_args(void);
 MN_API size_t mn_sizeof_rf_head(void);
 MN_API size_t mn_sizeof_llm(void);
@@ -751,6 +751,105 @@ MN_API int mn_stream_mfma_grouped_w8(const uint16_t* Y, int y_rows, const uint8_
 MN_API int mn_gemm256_f8(const uint8_t* A, int64_t lda, const float* a_scale, const uint8_t* W, int64_t ldw, const float* w_scale,
                          const uint16_t* bias, void* C, int64_t ldc, int M, int N, int K, int swiglu, int ksplit, void* stream);
 MN_API int mn_gemm256_f8_slices(int K, int ksplit);
+
+/* ------------------------------------------------------------------------------------------
+ * 9. Latent-cache sequence models (0.1.25): decoder stacks whose attention layers cache one low-rank latent per token instead of
+ *    keys and values (keys and values of every head are linear maps of it, so queries are absorbed into latent space and the
+ *    attention runs against the latents themselves), with a short causal per-channel filter in front of the mixer, sigmoid-gated
+ *    sublayer results that are normalised before the residual add, and a polynomial-of-unit-norms feed-forward activation.
+ *    Rows are fp32, weights bf16 [out, in]; every size and constant is a field or an argument.  The residual stream, norms,
+ *    gates, softmax and the cached latents are fp32 in both arithmetic modes; `arith` chooses the matrix products:
+ *    MN_SEQ_ARITH_BF16 = bf16 MFMA products with fp32 accumulation for steps of more than 8 rows (fp32 FMA below),
+ *    MN_SEQ_ARITH_F32 = fp32 FMA everywhere.
+ * ------------------------------------------------------------------------------------------ */
+MN_API int mn_affine_ln_rows(const float* x, int64_t ldx, const uint16_t* w, const uint16_t* b, float eps, float* y, int64_t ldy,
+                             uint16_t* y16, int64_t ldy16, int M, int n, void* stream);
+/* x += LN(sigmoid(g) * y; w, b) row by row (g holds the gate's pre-activation) */
+MN_API int mn_gated_ln_residual(float* x, int64_t ldx, const float* g, int64_t ldg, const float* y, int64_t ldy, const uint16_t* w,
+                                const uint16_t* b, float eps, int M, int n, void* stream);
+/* y = x / sqrt(mean(x^2) + eps) * w; with row_seq / row_slot the fp32 output row of input row m is row_seq[m] * t_max + row_slot[m]
+ * (append into a cache arena [n_seq, t_max, n]); y16 (optional) is a bf16 copy in input row order */
+MN_API int mn_rms_rows(const float* x, int64_t ldx, const uint16_t* w, float eps, float* y, int64_t ldy, uint16_t* y16, int64_t ldy16,
+                       const int32_t* row_seq, const int32_t* row_slot, int t_max, int M, int n, void* stream);
+/* y = c0 U(z) + c1 U(z^2) + c2 U(z^3) + c3 with U(v) = v / sqrt(mean(v^2) + eps), powers element by element; coef bf16 [4] */
+MN_API int mn_polynorm_rows(const float* z, int64_t ldz, const uint16_t* coef, float eps, float* y, int64_t ldy, uint16_t* y16,
+                            int64_t ldy16, int M, int n, void* stream);
+/* Causal per-channel filter over each sequence's rows, added to its input: y_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j), w bf16
+ * [n, taps].  Row m is position row_slot[m] of sequence row_seq[m] and has row_back[m] earlier rows of its sequence in this call
+ * (directly before it); older inputs come from state fp32 [n_seq, taps - 1, n] (entry i = the input i + 1 positions before the
+ * call's first row of that sequence), positions before 0 count as zero.  mn_tap_state_update moves the state past the call's rows. */
+MN_API int mn_tap_filter_rows(const float* x, int64_t ldx, const uint16_t* w, int taps, const float* state, const int32_t* row_seq,
+                              const int32_t* row_slot, const int32_t* row_back, float* y, int64_t ldy, uint16_t* y16, int64_t ldy16,
+                              int M, int n, void* stream);
+MN_API int mn_tap_state_update(const float* x, int64_t ldx, int taps, float* state, const int32_t* row_seq, const int32_t* row_back,
+                               int M, int n, void* stream);
+MN_API int mn_softcap_rows(float* z, int64_t ld, int M, int n, float cap, void* stream);
+/* C[z] = alpha * A[z] W[z]^T (+ bias) (* sigmoid(G[z])) for z < batch, operands of batch entry z at base + z * (their _bs stride):
+ * fp32 FMA, any M / N / K.  C (fp32) and C16 (bf16 copy) are both optional outputs. */
+MN_API int mn_gemm_f32_batched(const float* A, int64_t lda, int64_t a_bs, const uint16_t* W, int64_t ldw, int64_t w_bs,
+                               const uint16_t* bias, float* C, int64_t ldc, int64_t c_bs, uint16_t* C16, int64_t ldc16, int64_t c16_bs,
+                               const float* G, int64_t ldg, int64_t g_bs, int M, int N, int K, int batch, float alpha, void* stream);
+/* Attention against cached latents.  qabs fp32 [M, H, r]: the queries of every head mapped into latent space, softmax scale
+ * included; arena fp32 [n_seq, t_max, r]; row m attends slots [0, row_len[m]) of sequence row_seq[m].  blk_tab int32 [n_blk, 2] =
+ * (first row, rows <= mn_latent_attn_block_rows()) cuts the rows into runs of consecutive rows of ONE sequence with ascending
+ * row_len.  lat fp32 [M, H, r] = softmax-weighted mean of the latents.  ks > 1 splits the key range over ks workgroups per run
+ * (mn_latent_attn_splits proposes it from the launch size; workspace from mn_latent_attn_workspace_bytes).  r <= 512. */
+MN_API int mn_latent_attn_block_rows(void);
+MN_API int mn_latent_attn_splits(int n_blk, int max_len, int r);
+MN_API size_t mn_latent_attn_workspace_bytes(int M, int H, int r, int ks);
+MN_API int mn_latent_attn(const float* qabs, const float* arena, const int32_t* row_seq, const int32_t* row_len, const int32_t* blk_tab,
+                          int n_blk, int M, int H, int r, int t_max, int max_len, int ks, float* lat, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+enum { MN_SEQ_ARITH_BF16 = 0, MN_SEQ_ARITH_F32 = 1 };
+enum { MN_SEQ_MIX_LATENT_Q = 0,   /* queries through an RMS-normed latent (w_in rows: [q latent ; kv latent]) */
+       MN_SEQ_MIX_GATED = 1 };    /* direct queries, sigmoid gate on the concatenated heads (w_in rows: [q ; gate ; kv latent]) */
+typedef struct mn_seq_layer {
+  int32_t kind, heads, dim, vdim, kv_rank, q_rank; /* q_rank: MN_SEQ_MIX_LATENT_Q only */
+  int32_t ff;                                      /* 0: the layer has no feed-forward */
+  int32_t arena;                                   /* index of the latent arena it attends */
+  int32_t writes_arena;                            /* 1: w_in ends with its own kv-latent rows and it appends them; 0: it reads another layer's */
+  float scale;
+  const uint16_t *norm1_w, *norm1_b, *norm1b_w, *norm1b_b, *norm2_w, *norm2_b, *norm2b_w, *norm2b_b;   /* [width] each */
+  const uint16_t *taps_w;                          /* [width, taps] */
+  const uint16_t *rg1_w, *rg1_b;                   /* gate of the mixer's result: [width, width], [width] */
+  const uint16_t *w_in;                            /* the mixer's projections of its input, stacked by rows (see kind) */
+  const uint16_t *q_norm, *kv_norm;                /* [q_rank], [kv_rank] */
+  const uint16_t *w_uq;                            /* [heads * dim, q_rank] */
+  const uint16_t *w_ukT;                           /* [heads, kv_rank, dim]: the key expansion of every head, transposed */
+  const uint16_t *w_uv;                            /* [heads * vdim, kv_rank] */
+  const uint16_t *w_o;                             /* [width, heads * vdim] */
+  const uint16_t *w_ff_in, *b_ff_in;               /* [width + ff, width] = [feed-forward gate ; up], bias [width + ff] (zero on the up rows) */
+  const uint16_t *w_down;                          /* [width, ff] */
+  const uint16_t *act;                             /* [4] */
+} mn_seq_layer;
+typedef struct mn_seq_model {
+  int32_t width, n_layers, taps, arith;
+  float eps;
+  const mn_seq_layer* layers;                      /* HOST array [n_layers] */
+  const uint16_t *final_w, *final_b;
+} mn_seq_model;
+typedef struct mn_seq_state {
+  float* const* latent;                            /* HOST array of device pointers: arena a = fp32 [n_seq, t_max, its layer's kv_rank] */
+  float* taps;                                     /* fp32 [n_layers, n_seq, taps - 1, width] */
+  int32_t n_seq, t_max;
+} mn_seq_state;
+MN_API size_t mn_sizeof_seq_layer(void);
+MN_API size_t mn_sizeof_seq_model(void);
+MN_API size_t mn_sizeof_seq_state(void);
+/* One pass of the stack over M rows (a prefill portion, decode rows of several sequences, or a mix; each sequence's rows
+ * consecutive and in order).  x fp32 [M, width]: input embeddings.  Per row: row_seq (cache sequence), row_slot (its position =
+ * the cache slot its latent goes to), row_back (earlier rows of its sequence in this call), row_len (= row_slot + 1: slots it
+ * attends); blk_tab / n_blk as in mn_latent_attn; max_len >= every row_len.  Appends the latents, advances the filter states.
+ * out fp32 [M, width]: the final norm's output.  trace (optional) fp32 [n_layers, M, width]: the residual stream after every layer. */
+MN_API size_t mn_seq_workspace_bytes(const mn_seq_model* m, int M, int max_len);
+MN_API int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
+                       const int32_t* row_slot, const int32_t* row_back, const int32_t* row_len, const int32_t* blk_tab, int n_blk,
+                       int max_len, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
+/* logits fp32 [M, V] = hidden W^T by the step's product routing (arith as in mn_seq_model), then the soft cap (cap <= 0: none);
+ * workspace: M * K * 2 bytes (the bf16 operand of the MFMA route) */
+MN_API int mn_seq_logits(const float* hidden, int64_t ldh, int M, const uint16_t* W, int V, int K, float cap, int arith, float* out,
+                         int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

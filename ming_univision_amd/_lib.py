@@ -107,9 +107,27 @@ class LlmTp(C.Structure):
     ]
 
 
+class SeqLayer(C.Structure):
+    _fields_ = [(k, C.c_int32) for k in ("kind", "heads", "dim", "vdim", "kv_rank", "q_rank", "ff", "arena", "writes_arena")] + \
+               [("scale", C.c_float)] + \
+               [(k, C.c_void_p) for k in ("norm1_w", "norm1_b", "norm1b_w", "norm1b_b", "norm2_w", "norm2_b", "norm2b_w", "norm2b_b",
+                                          "taps_w", "rg1_w", "rg1_b", "w_in", "q_norm", "kv_norm", "w_uq", "w_ukT", "w_uv", "w_o",
+                                          "w_ff_in", "b_ff_in", "w_down", "act")]
+
+
+class SeqModel(C.Structure):
+    _fields_ = [("width", C.c_int32), ("n_layers", C.c_int32), ("taps", C.c_int32), ("arith", C.c_int32), ("eps", C.c_float),
+                ("layers", C.POINTER(SeqLayer)), ("final_w", C.c_void_p), ("final_b", C.c_void_p)]
+
+
+class SeqState(C.Structure):
+    _fields_ = [("latent", PP), ("taps", C.c_void_p), ("n_seq", C.c_int32), ("t_max", C.c_int32)]
+
+
 # (struct id of mn_struct_layout, its mn_sizeof_* export, the ctypes mirror): checked against the library at load time (`lib()`)
 STRUCTS = ((0, "mn_sizeof_skinny_args", SkinnyArgs), (1, "mn_sizeof_rf_head", RfHead), (2, "mn_sizeof_llm", Llm),
-           (3, "mn_sizeof_semdec", SemDec), (4, "mn_sizeof_tp_comm", TpComm), (5, "mn_sizeof_llm_tp", LlmTp))
+           (3, "mn_sizeof_semdec", SemDec), (4, "mn_sizeof_tp_comm", TpComm), (5, "mn_sizeof_llm_tp", LlmTp),
+           (6, "mn_sizeof_seq_layer", SeqLayer), (7, "mn_sizeof_seq_model", SeqModel), (8, "mn_sizeof_seq_state", SeqState))
 
 
 def check_struct_layouts(handle):
@@ -249,6 +267,23 @@ SYMBOLS = {
     "mn_lmhead_argmax": (_i, [_p, _i64, _i, _p, _i64, _i, _i, _i64, _p, _p, _p, _sz, _p]),
     "mn_sample_logits": (_i, [_p, _i64, _i, _i, _f, _i, _f, _p, _i64, _p, _p, _p]),
     "mn_semdec_workspace_bytes": (_sz, [C.POINTER(SemDec), _i, _i64]),
+    # section 9: latent-cache sequence models
+    "mn_sizeof_seq_layer": (_sz, []), "mn_sizeof_seq_model": (_sz, []), "mn_sizeof_seq_state": (_sz, []),
+    "mn_affine_ln_rows": (_i, [_p, _i64, _p, _p, _f, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_gated_ln_residual": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _f, _i, _i, _p]),
+    "mn_rms_rows": (_i, [_p, _i64, _p, _f, _p, _i64, _p, _i64, _p, _p, _i, _i, _i, _p]),
+    "mn_polynorm_rows": (_i, [_p, _i64, _p, _f, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_tap_filter_rows": (_i, [_p, _i64, _p, _i, _p, _p, _p, _p, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_tap_state_update": (_i, [_p, _i64, _i, _p, _p, _p, _i, _i, _p]),
+    "mn_softcap_rows": (_i, [_p, _i64, _i, _i, _f, _p]),
+    "mn_gemm_f32_batched": (_i, [_p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i, _i, _i, _i, _f, _p]),
+    "mn_latent_attn_block_rows": (_i, []),
+    "mn_latent_attn_splits": (_i, [_i, _i, _i]),
+    "mn_latent_attn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "mn_latent_attn": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _sz, _p]),
+    "mn_seq_workspace_bytes": (_sz, [C.POINTER(SeqModel), _i, _i]),
+    "mn_seq_step": (_i, [C.POINTER(SeqModel), C.POINTER(SeqState), _p, _i64, _i, _p, _p, _p, _p, _p, _i, _i, _p, _p, _p, _sz, _p]),
+    "mn_seq_logits": (_i, [_p, _i64, _i, _p, _i, _i, _f, _i, _p, _i64, _p, _sz, _p]),
     "mn_semdec_step": (_i, [C.POINTER(SemDec), _p, _i, _p, _p, _p, _p, _i, _i64, _p, _p, _p, _sz, _p]),
 }
 
@@ -269,7 +304,7 @@ def lib():
         fn = getattr(handle, name)  # AttributeError if the symbol is missing
         fn.restype = res
         fn.argtypes = args
-    if handle.mn_version() < 124:
+    if handle.mn_version() < 125:
         raise RuntimeError("libmingnative.so is too old")
     check_struct_layouts(handle)
     _lib = handle

@@ -5,6 +5,11 @@
   MingUniVisionConfig  <- mingunivision/configuration_bailingmm.py:20-31
                           (+ `vishead_diffloss_config`, asserted at modeling_bailingmm.py:118)
 
+  PizitarConfig        <- a decoder-only language model of latent-attention layers (no reference counterpart): config.json keys
+                          `architecture`, `width`, `vocab`, `layers`, `canon.taps`, `norm.eps`, `logit_softcap`
+
+`config_from_pretrained(dir)` picks the class by what config.json says (MODEL_REGISTRY).
+
 Plain Python (no transformers dependency): `from_dict` / `to_dict` /
 `from_json_file` / `from_pretrained(dir)` read the same JSON the reference's HF
 configs serialise to; unknown keys are kept as attributes like PretrainedConfig does.
@@ -292,3 +297,105 @@ def linear_proj_param_shapes(feature_dim, hidden_size, mlp_depth, prefix="linear
         s[prefix + f"{2 * i}.weight"] = (hidden_size, hidden_size)
         s[prefix + f"{2 * i}.bias"] = (hidden_size,)
     return s
+
+
+# ---- Pizitar ---------------------------------------------------------------------------------------------------------------
+PIZITAR_MIXERS = ("latent_attention", "latent_attention_2")
+
+
+class PizitarConfig(_Config):
+    """A stack of latent-attention layers.  `layers` is a list of dicts(type, mixer, mlp):
+    type  "latent_attention"   queries through an RMS-normed latent of `q_rank` rows; optional `kv_from`: j = attend layer j's cached
+                               latents (this layer then has no kv projection of its own)
+          "latent_attention_2" direct queries and a sigmoid gate on the concatenated heads
+    mixer heads, dim (query / key size per head), vdim, kv_rank (size of the cached latent), scale (of the scores)
+    mlp   None or dict(kind="dense", ff)
+    Every size is read from here or from the tensors; nothing is assumed equal between layers."""
+    model_type = "pizitar"
+
+    def __init__(self, width=256, vocab=1024, layers=(), canon=None, norm=None, logit_softcap=None, architecture="Pizitar", **kwargs):
+        self.architecture = architecture
+        self.width, self.vocab = int(width), int(vocab)
+        self.layers = [copy.deepcopy(dict(ly)) for ly in layers]
+        self.canon = dict(canon or {"taps": 1})
+        self.norm = dict(norm or {"eps": 1e-6})
+        self.logit_softcap = logit_softcap
+        super().__init__(**kwargs)
+        self.validate()
+
+    taps = property(lambda self: int(self.canon["taps"]))
+    eps = property(lambda self: float(self.norm["eps"]))
+
+    def validate(self):
+        if self.taps < 1:
+            raise ValueError("canon.taps must be >= 1")
+        for i, ly in enumerate(self.layers):
+            if ly.get("type") not in PIZITAR_MIXERS:
+                raise ValueError(f"layer {i}: unknown mixer type {ly.get('type')!r} (known: {PIZITAR_MIXERS})")
+            m = ly["mixer"]
+            for k in ("heads", "dim", "vdim", "kv_rank", "scale"):
+                if k not in m:
+                    raise ValueError(f"layer {i}: mixer lacks {k!r}")
+            if ly["type"] == "latent_attention" and "q_rank" not in m:
+                raise ValueError(f"layer {i}: latent_attention needs q_rank")
+            src = m.get("kv_from")
+            if src is not None:
+                if ly["type"] != "latent_attention":
+                    raise ValueError(f"layer {i}: kv_from is a latent_attention option")
+                if not (0 <= src < i) or self.layers[src]["mixer"].get("kv_from") is not None:
+                    raise ValueError(f"layer {i}: kv_from = {src} must name an earlier layer that projects its own latent")
+                if self.layers[src]["mixer"]["kv_rank"] != m["kv_rank"]:
+                    raise ValueError(f"layer {i}: kv_rank differs from layer {src}'s, whose latents it attends")
+            mlp = ly.get("mlp")
+            if mlp is not None and mlp.get("kind") != "dense":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+
+
+def pizitar_param_shapes(cfg: PizitarConfig):
+    """{tensor name: shape} of a Pizitar checkpoint (`l<i>.` per layer; `.b` = the bias of the tensor it follows)."""
+    W, V, taps = cfg.width, cfg.vocab, cfg.taps
+    s = {"embed": (V, W)}
+    for i, ly in enumerate(cfg.layers):
+        p, m, mlp = f"l{i}.", ly["mixer"], ly.get("mlp")
+        H, d, v, r = m["heads"], m["dim"], m["vdim"], m["kv_rank"]
+        for n in ("norm1", "norm1b") + (("norm2", "norm2b") if mlp is not None else ()):
+            s[p + n], s[p + n + ".b"] = (W,), (W,)
+        if ly["type"] == "latent_attention":
+            s[p + "mix.dq"], s[p + "mix.dq.norm"], s[p + "mix.uq"] = (m["q_rank"], W), (m["q_rank"],), (H * d, m["q_rank"])
+        else:
+            s[p + "mix.q"], s[p + "mix.g"] = (H * d, W), (H * v, W)
+        if m.get("kv_from") is None:
+            s[p + "mix.dkv"], s[p + "mix.dkv.norm"] = (r, W), (r,)
+        s[p + "mix.uk"], s[p + "mix.uv"], s[p + "mix.o"] = (H * d, r), (H * v, r), (W, H * v)
+        if mlp is not None:
+            s[p + "mlp.up"], s[p + "mlp.down"], s[p + "mlp.act"] = (mlp["ff"], W), (W, mlp["ff"]), (4,)
+            s[p + "rg2"], s[p + "rg2.b"] = (W, W), (W,)
+        s[p + "canon1"] = (W, taps)
+        s[p + "rg1"], s[p + "rg1.b"] = (W, W), (W,)
+    s["final.norm"], s["final.norm.b"], s["head"] = (W,), (W,), (V, W)
+    return s
+
+
+# ---- registry: which configuration class a config.json belongs to -------------------------------------------------------------
+def _is_pizitar(d):
+    return d.get("architecture") == "Pizitar" or d.get("model_type") == "pizitar"
+
+
+def _is_ming_univision(d):
+    return "llm_config" in d or d.get("model_type") in ("bailingmm", "ming_univision")
+
+
+MODEL_REGISTRY = [("pizitar", _is_pizitar, PizitarConfig), ("ming_univision", _is_ming_univision, MingUniVisionConfig)]
+
+
+def config_from_pretrained(path):
+    """-> (registry name, configuration) of the model in `path` (a directory with config.json, or the file itself)."""
+    if os.path.isdir(path):
+        path = os.path.join(path, "config.json")
+    with open(path) as f:
+        d = json.load(f)
+    for name, match, klass in MODEL_REGISTRY:
+        if match(d):
+            return name, klass.from_dict(d)
+    raise ValueError(f"{path}: no model of this framework matches (architecture = {d.get('architecture')!r}, "
+                     f"model_type = {d.get('model_type')!r}); known: {[n for n, _, _ in MODEL_REGISTRY]}")

@@ -112,10 +112,29 @@ extern "C" int mn_struct_layout(int which, size_t* offsets, int cap) {
       F(expert0) F(n_local_experts) F(shared_inter) F(ws_gate_up) F(ws_down) F(ws_gate_up_scale) F(ws_down_scale)
 #undef F
   };
-  const size_t* tab[] = {skinny, rf, llm, semdec, comm, llm_tp};
+  static const size_t seq_layer[] = {
+#define F(f) MN_OFF(mn_seq_layer, f)
+      F(kind) F(heads) F(dim) F(vdim) F(kv_rank) F(q_rank) F(ff) F(arena) F(writes_arena) F(scale) F(norm1_w) F(norm1_b) F(norm1b_w)
+      F(norm1b_b) F(norm2_w) F(norm2_b) F(norm2b_w) F(norm2b_b) F(taps_w) F(rg1_w) F(rg1_b) F(w_in) F(q_norm) F(kv_norm) F(w_uq) F(w_ukT)
+      F(w_uv) F(w_o) F(w_ff_in) F(b_ff_in) F(w_down) F(act)
+#undef F
+  };
+  static const size_t seq_model[] = {
+#define F(f) MN_OFF(mn_seq_model, f)
+      F(width) F(n_layers) F(taps) F(arith) F(eps) F(layers) F(final_w) F(final_b)
+#undef F
+  };
+  static const size_t seq_state[] = {
+#define F(f) MN_OFF(mn_seq_state, f)
+      F(latent) F(taps) F(n_seq) F(t_max)
+#undef F
+  };
+  const size_t* tab[] = {skinny, rf, llm, semdec, comm, llm_tp, seq_layer, seq_model, seq_state};
   const int cnt[] = {(int)(sizeof(skinny) / sizeof(size_t)), (int)(sizeof(rf) / sizeof(size_t)), (int)(sizeof(llm) / sizeof(size_t)),
-                     (int)(sizeof(semdec) / sizeof(size_t)), (int)(sizeof(comm) / sizeof(size_t)), (int)(sizeof(llm_tp) / sizeof(size_t))};
-  MN_CHECK_ARG(which >= 0 && which < 6, "mn_struct_layout: unknown struct id");
+                     (int)(sizeof(semdec) / sizeof(size_t)), (int)(sizeof(comm) / sizeof(size_t)), (int)(sizeof(llm_tp) / sizeof(size_t)),
+                     (int)(sizeof(seq_layer) / sizeof(size_t)), (int)(sizeof(seq_model) / sizeof(size_t)),
+                     (int)(sizeof(seq_state) / sizeof(size_t))};
+  MN_CHECK_ARG(which >= 0 && which < 9, "mn_struct_layout: unknown struct id");
   for (int i = 0; i < cnt[which] && i < cap; ++i) offsets[i] = tab[which][i];
   return cnt[which];
 }
