@@ -793,7 +793,7 @@ MN_API int mn_gemm_f32_batched(const float* A, int64_t lda, int64_t a_bs, const 
  * included; arena fp32 [n_seq, t_max, r]; row m attends slots [0, row_len[m]) of sequence row_seq[m].  blk_tab int32 [n_blk, 2] =
  * (first row, rows <= mn_latent_attn_block_rows()) cuts the rows into runs of consecutive rows of ONE sequence with ascending
  * row_len.  lat fp32 [M, H, r] = softmax-weighted mean of the latents.  ks > 1 splits the key range over ks workgroups per run
- * (mn_latent_attn_splits proposes it from the launch size; workspace from mn_latent_attn_workspace_bytes).  r <= 512. */
+ * (mn_latent_attn_splits proposes it from the launch size; workspace from mn_latent_attn_workspace_bytes).  r <= 1024. */
 MN_API int mn_latent_attn_block_rows(void);
 MN_API int mn_latent_attn_splits(int n_blk, int max_len, int r);
 MN_API size_t mn_latent_attn_workspace_bytes(int M, int H, int r, int ks);

@@ -407,7 +407,7 @@ extern "C" int mn_gemm_f32_batched(const float* A, int64_t lda, int64_t a_bs, co
 
 // rows of a workgroup (consecutive rows of one sequence) and the key-tile length for latent size r
 extern "C" int mn_latent_attn_block_rows(void) { return 4; }
-static inline int latent_kt(int r) { return r <= 256 ? 64 : 32; }
+static inline int latent_kt(int r) { return r <= 256 ? 64 : r <= 512 ? 32 : 16; }   // the tile [KT][r + 1] fp32 stays below 66 KiB
 
 extern "C" int mn_latent_attn_splits(int n_blk, int max_len, int r) {
   const int KT = latent_kt(r);
@@ -428,7 +428,7 @@ extern "C" int mn_latent_attn(const float* qabs, const float* arena, const int32
                               void* stream) {
   MN_CHECK_ARG(qabs && arena && row_seq && row_len && blk_tab && lat && n_blk >= 1 && M >= 1 && H >= 1 && r >= 1 && t_max >= 1,
                "mn_latent_attn: bad args");
-  MN_CHECK_ARG(r <= 512, "mn_latent_attn: latent size %d above 512 is not supported", r);
+  MN_CHECK_ARG(r <= 1024, "mn_latent_attn: latent size %d above 1024 is not supported", r);
   MN_CHECK_ARG(max_len >= 1 && max_len <= t_max && ks >= 1 && ks <= 65535, "mn_latent_attn: bad max_len=%d / ks=%d", max_len, ks);
   MN_CHECK_ARG(ws_bytes >= mn_latent_attn_workspace_bytes(M, H, r, ks) && (ks == 1 || ws), "mn_latent_attn: workspace too small");
   const int KT = latent_kt(r), RB = mn_latent_attn_block_rows();
@@ -450,7 +450,7 @@ extern "C" int mn_latent_attn(const float* qabs, const float* arena, const int32
     hipLaunchKernelGGL((latent_attn_kernel<R_>), grid, block, lds, st, qabs, arena, row_seq, row_len, blk_tab, H, r, t_max, KT, tps, lat, \
                        pacc, pml, ks, M);                                                                                           \
   } while (0)
-  if (r <= 64) MN_LA(1); else if (r <= 128) MN_LA(2); else if (r <= 256) MN_LA(4); else MN_LA(8);
+  if (r <= 64) MN_LA(1); else if (r <= 128) MN_LA(2); else if (r <= 256) MN_LA(4); else if (r <= 512) MN_LA(8); else MN_LA(16);
 #undef MN_LA
   MN_CHECK_LAUNCH("mn_latent_attn");
   if (ks > 1) {
