@@ -244,9 +244,10 @@ __global__ __launch_bounds__(1024) void latent_attn_kernel(const float* __restri
   for (int tile = t0; tile < t1; ++tile) {
     const int key0 = tile * KT;
     __syncthreads();
-    for (int e = threadIdx.x; e < KT * r; e += blockDim.x) {
-      const int j = e / r, d = e - j * r;
-      lds_c[j * ldc + d] = (key0 + j < len_max) ? arena[(seq * t_max + key0 + j) * r + d] : 0.f;
+    for (int j = wave; j < KT; j += NW) {            // a wave copies whole latent rows: consecutive lanes, consecutive components
+      const bool in = key0 + j < len_max;
+      const float* src = arena + (seq * t_max + key0 + j) * r;
+      for (int d = lane; d < r; d += 64) lds_c[j * ldc + d] = in ? src[d] : 0.f;
     }
     __syncthreads();
     if (!active || key0 >= my_len) continue;
@@ -413,7 +414,7 @@ extern "C" int mn_latent_attn_splits(int n_blk, int max_len, int r) {
   const int KT = latent_kt(r);
   const int tiles = (int)mn_cdiv(max_len > 0 ? max_len : 1, KT);
   int ks = (int)mn_cdiv(2 * (int64_t)mn_num_cus(), n_blk > 0 ? n_blk : 1);
-  const int cap = (int)mn_cdiv(tiles, 4);              // a split works on at least 4 key tiles
+  const int cap = (int)mn_cdiv(tiles, 2);              // a split works on at least 2 key tiles
   if (ks > cap) ks = cap;
   if (ks > 64) ks = 64;
   return ks < 1 ? 1 : ks;

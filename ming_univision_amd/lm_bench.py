@@ -1,0 +1,157 @@
+"""Prefill / decode throughput of the Pizitar decoder beside the Bailing-MoE decoder at equal size (`bench.py --lm-compare`).
+
+Random weights at sizes that resemble real layers.  "Equal size": same width, depth and head count, 128-wide heads on both, and a
+feed-forward whose ACTIVE hidden width matches (the MoE runs 8 experts, top-2, of half the dense hidden width each).  Both run
+their serving paths: Pizitar `forward_spans` / `step` (bf16 arithmetic), Bailing-MoE `prefill_mfma` (its bf16 regime) and `step`.
+Beside the end-to-end rates the attention kernels are timed alone against their rooflines — what each must move or multiply:
+  decode   bytes of cache read per step / HBM peak        (latents [len, r] fp32  vs  keys + values [len, n_kv, 128] x 2 fp32)
+  prefill  multiply-adds of the causal score / value products at the precision the kernel runs them
+           (fp32 FMA peak for the latent kernel, bf16 MFMA peak for the flash kernel)
+"""
+import time
+
+import torch
+
+HBM_GBS = 8000.0
+MFMA_BF16_TFLOPS = 2500.0
+FMA_F32_TFLOPS = 157.3
+
+SIZES = {
+    "w1024": dict(width=1024, layers=4, heads=8, kv_rank=256, q_rank=384, ff=4096, vocab=32000),
+    "w2048": dict(width=2048, layers=4, heads=16, kv_rank=512, q_rank=768, ff=8192, vocab=32000),
+}
+
+
+def _time(fn, iters, warm=2):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / iters
+
+
+def pizitar_config(s):
+    from .configuration import PizitarConfig
+    la = dict(type="latent_attention", mixer=dict(heads=s["heads"], dim=128, vdim=128, kv_rank=s["kv_rank"], q_rank=s["q_rank"], scale=128 ** -0.5),
+              mlp=dict(kind="dense", ff=s["ff"]))
+    lb = dict(type="latent_attention_2", mixer=dict(heads=s["heads"], dim=128, vdim=128, kv_rank=s["kv_rank"], scale=128 ** -0.5),
+              mlp=dict(kind="dense", ff=s["ff"]))
+    return PizitarConfig(width=s["width"], vocab=s["vocab"], layers=[la, lb] * (s["layers"] // 2), canon=dict(taps=4), norm=dict(eps=1e-6),
+                         logit_softcap=30.0)
+
+
+def bailing_config(s):
+    from .configuration import BailingMoeConfig
+    return BailingMoeConfig(vocab_size=s["vocab"], hidden_size=s["width"], num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
+                            num_key_value_heads=s["heads"] // 4, head_dim=128, use_bias=False, use_qkv_bias=False, rope_theta=600000.0,
+                            num_experts=8, num_shared_experts=0, num_experts_per_tok=2, moe_intermediate_size=s["ff"] // 2, multi_gate=False,
+                            first_k_dense_replace=0, norm_topk_prob=True)
+
+
+def run_pizitar(s, T, batches, n_dec):
+    from ._lib import check, current_stream, lib, ptr
+    from .pizitar import PizitarDecoder
+    dev = "cuda"
+    cfg = pizitar_config(s)
+    dec = PizitarDecoder.synthetic(cfg, dev, t_max=T + n_dec + 8, n_seq=max(batches), arith="bf16")
+    ids = torch.randint(0, s["vocab"], (T,), device=dev)
+    x = dec.embed(ids)
+    out = {"prefill_tokens_per_s": T / _time(lambda: dec.forward_spans(x, [(0, T, 0)]), 3)}
+    for B in batches:
+        for b in range(1, B):
+            for a in dec.latent:
+                a[b, :T] = a[0, :T]
+            dec.taps_state[:, b] = dec.taps_state[:, 0]
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        back, blk = dec.decode_tables(B)
+        xb = dec.embed(torch.randint(0, s["vocab"], (B,), device=dev))
+
+        def loop():
+            slot = torch.full((B,), T, dtype=torch.int32, device=dev)
+            ln = slot + 1
+            for i in range(n_dec):
+                dec.step(xb, row_seq, slot, back, ln, blk, T + i + 1)
+                check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
+        out[f"decode_b{B}_tokens_per_s"] = B * n_dec / _time(loop, 2, 1)
+    # the attention kernel alone
+    H, r = s["heads"], s["kv_rank"]
+    tabs = {k: (torch.from_numpy(v).to(dev) if k != "max_len" else v) for k, v in
+            __import__("ming_univision_amd.sequences", fromlist=["x"]).rows_of_spans([(0, T, 0)], dec.block_rows).items()}
+    q = torch.randn(T, H, r, device=dev) * 0.05
+    lat = torch.empty_like(q)
+    nb = tabs["blk_tab"].shape[0]
+    ks = lib().mn_latent_attn_splits(nb, T, r)
+    ws = torch.empty(max(16, lib().mn_latent_attn_workspace_bytes(T, H, r, ks)), dtype=torch.uint8, device=dev)
+    t = _time(lambda: check(lib().mn_latent_attn(ptr(q), ptr(dec.latent[0]), ptr(tabs["row_seq"]), ptr(tabs["row_len"]), ptr(tabs["blk_tab"]), nb,
+                                                 T, H, r, dec.t_max, T, ks, ptr(lat), ptr(ws), ws.numel(), current_stream())), 5)
+    flops = 2 * 2 * H * r * T * (T + 1) / 2
+    out["attn_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / FMA_F32_TFLOPS, peak="fp32 FMA")
+    for B in batches:
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        ln = torch.full((B,), T, dtype=torch.int32, device=dev)
+        _, blk = dec.decode_tables(B)
+        ks = lib().mn_latent_attn_splits(B, T, r)
+        ws = torch.empty(max(16, lib().mn_latent_attn_workspace_bytes(B, H, r, ks)), dtype=torch.uint8, device=dev)
+        t = _time(lambda: check(lib().mn_latent_attn(ptr(q), ptr(dec.latent[0]), ptr(row_seq), ptr(ln), ptr(blk), B, B, H, r, dec.t_max, T, ks,
+                                                     ptr(lat), ptr(ws), ws.numel(), current_stream())), 20)
+        byts = B * T * r * 4
+        out[f"attn_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS, key_splits=ks)
+    return out
+
+
+def run_bailing(s, T, batches, n_dec):
+    from . import ops
+    from ._lib import check, current_stream, lib, ptr
+    from .bailing_moe import BailingMoeDecoder
+    dev = "cuda"
+    cfg = bailing_config(s)
+    dec = BailingMoeDecoder.synthetic(cfg, dev, t_max=T + n_dec + 8, n_seq=max(batches))
+    ids = torch.randint(0, s["vocab"], (T,), device=dev)
+    x = dec.embed(ids)
+    out = {"prefill_tokens_per_s": T / _time(lambda: dec.prefill_mfma(x, seq=0), 3),
+           "prefill_fp32class_tokens_per_s": T / _time(lambda: dec.prefill_wide(x, seq=0), 3)}
+    for B in batches:
+        for b in range(1, B):
+            dec.copy_sequence(0, b, T)
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        xb = dec.embed(torch.randint(0, s["vocab"], (B,), device=dev))
+
+        def loop():
+            slot = torch.full((B,), T, dtype=torch.int32, device=dev)
+            ln = slot + 1
+            for i in range(n_dec):
+                dec.step(xb, row_seq, slot, slot, ln, distinct_sequences=True)
+                check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
+        out[f"decode_b{B}_tokens_per_s"] = B * n_dec / _time(loop, 2, 1)
+    nq, nkv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, 128
+    kv = dec.kv_cache[0]
+    for B in batches:
+        q = torch.randn(B, nq * hd, device=dev) * 0.05
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        ln = torch.full((B,), T, dtype=torch.int32, device=dev)
+        t = _time(lambda: ops.attn_decode(q, nq, nkv, hd, kv, row_seq, ln), 20)
+        byts = B * T * nkv * hd * 2 * 4
+        out[f"attn_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS)
+    # flash prefill alone (bf16 queries against the fp32 arena), one span of T rows
+    qb = (torch.randn(T, nq * hd, device=dev) * 0.05).to(torch.bfloat16)
+    att = torch.empty_like(qb)
+    tab = torch.tensor([[0, 0, T]], dtype=torch.int32, device=dev)
+    t = _time(lambda: check(lib().mn_flash_prefill_gqa_hd128(ptr(qb), ptr(kv), dec.t_max, nq, nkv, 0, ptr(tab), 1, T, None, 0, ptr(att),
+                                                             current_stream())), 5)
+    flops = 2 * 2 * nq * hd * T * (T + 1) / 2
+    out["attn_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / MFMA_BF16_TFLOPS, peak="bf16 MFMA")
+    return out
+
+
+def compare(sizes=("w1024", "w2048"), prompt=2048, batches=(1, 32), n_dec=32):
+    res = {}
+    for name in sizes:
+        s = SIZES[name]
+        torch.cuda.empty_cache()
+        res[name] = dict(size=s, prompt=prompt, pizitar=run_pizitar(s, prompt, batches, n_dec))
+        torch.cuda.empty_cache()
+        res[name]["bailing_moe"] = run_bailing(s, prompt, batches, n_dec)
+    return res
