@@ -800,6 +800,13 @@ MN_API size_t mn_latent_attn_workspace_bytes(int M, int H, int r, int ks);
 MN_API int mn_latent_attn(const float* qabs, const float* arena, const int32_t* row_seq, const int32_t* row_len, const int32_t* blk_tab,
                           int n_blk, int M, int H, int r, int t_max, int max_len, int ks, float* lat, void* workspace,
                           size_t workspace_bytes, void* stream);
+/* The same with the kernel named: MN_LATENT_ATTN_MFMA (what mn_latent_attn runs) = scores and weighted sums on the fp32 matrix
+ * cores (v_mfma_f32_16x16x4_f32: fp32 operands and accumulation), 16 query vectors per workgroup, 16-key tiles;
+ * MN_LATENT_ATTN_VALU = one wave per query vector on fp32 FMA (the plain kernel the other is checked against). */
+enum { MN_LATENT_ATTN_MFMA = 0, MN_LATENT_ATTN_VALU = 1 };
+MN_API int mn_latent_attn_ex(const float* qabs, const float* arena, const int32_t* row_seq, const int32_t* row_len, const int32_t* blk_tab,
+                             int n_blk, int M, int H, int r, int t_max, int max_len, int ks, float* lat, void* workspace,
+                             size_t workspace_bytes, int variant, void* stream);
 
 enum { MN_SEQ_ARITH_BF16 = 0, MN_SEQ_ARITH_F32 = 1 };
 enum { MN_SEQ_MIX_LATENT_Q = 0,   /* queries through an RMS-normed latent (w_in rows: [q latent ; kv latent]) */

@@ -281,6 +281,7 @@ SYMBOLS = {
     "mn_latent_attn_splits": (_i, [_i, _i, _i]),
     "mn_latent_attn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mn_latent_attn": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _sz, _p]),
+    "mn_latent_attn_ex": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _sz, _i, _p]),
     "mn_seq_workspace_bytes": (_sz, [C.POINTER(SeqModel), _i, _i]),
     "mn_seq_step": (_i, [C.POINTER(SeqModel), C.POINTER(SeqState), _p, _i64, _i, _p, _p, _p, _p, _p, _i, _i, _p, _p, _p, _sz, _p]),
     "mn_seq_logits": (_i, [_p, _i64, _i, _p, _i, _i, _f, _i, _p, _i64, _p, _sz, _p]),

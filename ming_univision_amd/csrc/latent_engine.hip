@@ -33,6 +33,12 @@ int linear(int arith, int M, const float* A, int64_t lda, const uint16_t* A16, i
   return mn_gemm_f32_batched(A, lda, 0, W, K, 0, bias, C, ldc, 0, nullptr, 0, 0, nullptr, 0, 0, M, N, K, 1, 1.0f, stream);
 }
 
+// the step's own copy of its input rows (a kernel, not a memcpy node: the step may be captured into a graph)
+__global__ void copy_rows_kernel(const float* __restrict__ x, int64_t ldx, float* __restrict__ y, int n) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c < n) y[(int64_t)blockIdx.y * n + c] = x[(int64_t)blockIdx.y * ldx + c];
+}
+
 struct Dims {
   int n_in, hd, hv, hr, q_rank, ff;
 };
@@ -133,10 +139,8 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
   hipStream_t hs = mn_stream(stream);
   int rc;
 #define MN_TRY(call) do { rc = (call); if (rc != MN_OK) return rc; } while (0)
-  {
-    const hipError_t e = hipMemcpy2DAsync(xr, (size_t)W * 4, x, (size_t)ldx * 4, (size_t)W * 4, R, hipMemcpyDeviceToDevice, hs);
-    if (e != hipSuccess) { mn_set_error("mn_seq_step: copy of the input rows: %s", hipGetErrorString(e)); return MN_ELAUNCH; }
-  }
+  hipLaunchKernelGGL(copy_rows_kernel, dim3((unsigned)mn_cdiv(W, 256), (unsigned)M), dim3(256), 0, hs, x, ldx, xr, W);
+  MN_CHECK_LAUNCH("mn_seq_step(copy)");
   const size_t taps_layer = (size_t)st->n_seq * (m->taps - 1) * W;
   for (int li = 0; li < m->n_layers; ++li) {
     const mn_seq_layer& l = m->layers[li];

@@ -102,6 +102,93 @@ __global__ __launch_bounds__(256) void polynorm_kernel(const float* __restrict__
   }
 }
 
+// One workgroup per row with the row held in registers (VPT values per thread, n <= 256 VPT): one batch of loads, the reductions,
+// one batch of stores — the form for wide rows, where a single wave walking the row three times is a chain of dependent round trips.
+enum { ROW_LN = 0, ROW_GATED_LN_RESIDUAL = 1, ROW_POLYNORM = 2 };
+struct RowArgs {
+  const float* x; int64_t ldx;          // LN / polynorm input; gated: the residual stream (updated in place)
+  const float* g; int64_t ldg;          // gated: gate pre-activation
+  const float* y; int64_t ldy;          // gated: sublayer result
+  const bf16_t* w; const bf16_t* b;     // norm weight / bias; polynorm: w = the four coefficients
+  float eps;
+  float* out; int64_t ldo;
+  bf16_t* out16; int64_t ldo16;
+  int n;
+};
+
+template <int VPT, int MODE>
+__global__ __launch_bounds__(256) void row_block_kernel(RowArgs a) {
+  __shared__ float red[8];
+  const int row = blockIdx.x, tid = threadIdx.x, n = a.n;
+  float v[VPT];
+  if (MODE == ROW_GATED_LN_RESIDUAL) {
+    float gv[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = tid + 256 * i, cc = c < n ? c : 0;
+      gv[i] = a.g[(int64_t)row * a.ldg + cc];
+      v[i] = a.y[(int64_t)row * a.ldy + cc];
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) v[i] = (tid + 256 * i < n) ? sigmoid_f(gv[i]) * v[i] : 0.f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = tid + 256 * i;
+      const float t = a.x[(int64_t)row * a.ldx + (c < n ? c : 0)];
+      v[i] = c < n ? t : 0.f;
+    }
+  }
+  if (MODE == ROW_POLYNORM) {
+    float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) { const float v2 = v[i] * v[i], v3 = v2 * v[i]; s2 += v2; s4 += v2 * v2; s6 += v3 * v3; }
+    s2 = block_sum(s2, red); s4 = block_sum(s4, red); s6 = block_sum(s6, red);
+    const float ca = bf16_to_f32(a.w[0]) / sqrtf(s2 / (float)n + a.eps), cb = bf16_to_f32(a.w[1]) / sqrtf(s4 / (float)n + a.eps),
+                cc = bf16_to_f32(a.w[2]) / sqrtf(s6 / (float)n + a.eps), ce = bf16_to_f32(a.w[3]);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = tid + 256 * i;
+      if (c >= n) continue;
+      const float v2 = v[i] * v[i], o = ca * v[i] + cb * v2 + cc * (v2 * v[i]) + ce;
+      if (a.out) a.out[(int64_t)row * a.ldo + c] = o;
+      if (a.out16) a.out16[(int64_t)row * a.ldo16 + c] = f32_to_bf16(o);
+    }
+    return;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) s += v[i];
+  const float mean = block_sum(s, red) / (float)n;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) { const float d = (tid + 256 * i < n) ? v[i] - mean : 0.f; q += d * d; }
+  const float rstd = 1.0f / sqrtf(block_sum(q, red) / (float)n + a.eps);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = tid + 256 * i;
+    if (c >= n) continue;
+    const float o = (v[i] - mean) * rstd * bf16_to_f32(a.w[c]) + bf16_to_f32(a.b[c]);
+    if (MODE == ROW_GATED_LN_RESIDUAL) {
+      a.out[(int64_t)row * a.ldo + c] += o;
+    } else {
+      if (a.out) a.out[(int64_t)row * a.ldo + c] = o;
+      if (a.out16) a.out16[(int64_t)row * a.ldo16 + c] = f32_to_bf16(o);
+    }
+  }
+}
+
+// rows of 512 .. 8192 values take the register form; launches it and returns true, or false for other widths
+template <int MODE>
+bool launch_row_block(const RowArgs& a, int M, hipStream_t st) {
+  if (a.n < 512 || a.n > 8192) return false;
+  const int vpt = (a.n + 255) / 256;
+#define MN_RB(V_) hipLaunchKernelGGL((row_block_kernel<V_, MODE>), dim3((unsigned)M), dim3(256), 0, st, a)
+  if (vpt <= 2) MN_RB(2); else if (vpt <= 4) MN_RB(4); else if (vpt <= 8) MN_RB(8); else if (vpt <= 16) MN_RB(16); else MN_RB(32);
+#undef MN_RB
+  return true;
+}
+
 // y[m, c] = x[m, c] + sum_k w[c, taps - 1 - k] * (the sequence's input k positions back); grid (ceil(n / 256), M)
 __global__ __launch_bounds__(256) void tap_filter_kernel(const float* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int taps,
                                                          const float* __restrict__ state, const int32_t* __restrict__ row_seq,
@@ -211,6 +298,35 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 a) {
   }
 }
 
+// C[z][m, n] = alpha * A[z][m, :] . W[z][n, :] (+ bias) (* sigmoid(G)) for M <= 8 rows: one wave per output column, lanes over K
+template <int MM>
+__global__ __launch_bounds__(256) void gemv_f32_kernel(GemmF32 a) {
+  const int z = blockIdx.z, n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (n >= a.N) return;
+  const float* A = a.A + (int64_t)z * a.a_bs;
+  const bf16_t* Wr = a.W + (int64_t)z * a.w_bs + (int64_t)n * a.ldw;
+  float acc[MM];
+#pragma unroll
+  for (int m = 0; m < MM; ++m) acc[m] = 0.f;
+#pragma unroll 4
+  for (int k = lane; k < a.K; k += 64) {
+    const float w = bf16_to_f32(Wr[k]);
+#pragma unroll
+    for (int m = 0; m < MM; ++m)
+      if (m < a.M) acc[m] = fmaf(A[(int64_t)m * a.lda + k], w, acc[m]);
+  }
+#pragma unroll
+  for (int m = 0; m < MM; ++m) {
+    if (m >= a.M) break;
+    float v = wave_sum(acc[m]) * a.alpha;
+    if (lane != 0) continue;
+    if (a.bias) v += bf16_to_f32(a.bias[n]);
+    if (a.G) v *= sigmoid_f(a.G[(int64_t)z * a.g_bs + (int64_t)m * a.ldg + n]);
+    if (a.C) a.C[(int64_t)z * a.c_bs + (int64_t)m * a.ldc + n] = v;
+    if (a.C16) a.C16[(int64_t)z * a.c16_bs + (int64_t)m * a.ldc16 + n] = f32_to_bf16(v);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------------------------
 // Latent attention.  One wave per query vector (row, head); the waves of a workgroup share the staged latent tile (all heads and up
 // to 4 consecutive rows of one sequence see the same keys).  Phase A: lane = key, dot over r; phase B: lane = latent component,
@@ -300,26 +416,171 @@ __global__ __launch_bounds__(1024) void latent_attn_kernel(const float* __restri
   }
 }
 
-// one wave per (row, head): combine the key splits
+// ---------------------------------------------------------------------------------------------------------------------------
+// Latent attention on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: fp32 operands, fp32 accumulate — scores and weights stay
+// 32-bit).  A workgroup of 4 waves owns 16 query vectors (row, head) of one run of rows and walks the sequence's latents in tiles
+// of 16 keys staged in LDS:
+//   scores   S[16 q, 16 keys] = Q C^T: every wave multiplies its quarter of the latent components, the partial tiles are summed
+//            through LDS, so all four waves hold the same scores and keep the same running maximum / sum without talking
+//   values   O[16 q, r] += P C: the weights go through LDS into the A-operand layout, wave w owns the 16-column blocks w, w + 4, ..
+// Operand layouts (lane l, c = l % 16, g = l / 16): A[row c][k g], B[k g][col c], D[row 4 g + i][col c] in VGPR i.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// 16 rows x 64 NBW floats, global -> registers -> LDS (row stride LDC), zero beyond n: 16 threads per row, 16 bytes per thread and
+// pass, every load of the tile in flight together.  row_ptr(j) must be readable for every j (callers clamp), row_ok(j) says whether
+// row j counts.  Split in two so that the next tile's loads fly while the current tile is multiplied.
+template <int NBW, typename RowPtr, typename RowOk>
+__device__ __forceinline__ void load16(f32x4 (&v)[NBW], int n, int tid, RowPtr row_ptr, RowOk row_ok) {
+  const int j = tid >> 4, cg = tid & 15;
+  const float* src = row_ptr(j);
+  const bool ok = row_ok(j);
+  if ((n & 3) == 0) {
+#pragma unroll
+    for (int ps = 0; ps < NBW; ++ps) {
+      const int d = 4 * (cg + 16 * ps);
+      const f32x4 t = *reinterpret_cast<const f32x4*>(src + (d < n ? d : 0));
+      v[ps] = (ok && d < n) ? t : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  } else {
+#pragma unroll
+    for (int ps = 0; ps < NBW; ++ps) {
+      const int d = 4 * (cg + 16 * ps);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float t = src[d + e < n ? d + e : 0];
+        v[ps][e] = (ok && d + e < n) ? t : 0.f;
+      }
+    }
+  }
+}
+template <int NBW, int LDC>
+__device__ __forceinline__ void store16(float* __restrict__ dst, const f32x4 (&v)[NBW], int tid) {
+  const int j = tid >> 4, cg = tid & 15;
+#pragma unroll
+  for (int ps = 0; ps < NBW; ++ps) *reinterpret_cast<f32x4*>(dst + j * LDC + 4 * (cg + 16 * ps)) = v[ps];
+}
+
+template <int NBW>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __restrict__ qabs, const float* __restrict__ arena,
+                                                               const int32_t* __restrict__ row_seq, const int32_t* __restrict__ row_len,
+                                                               const int32_t* __restrict__ blk_tab, int H, int r, int t_max,
+                                                               int tiles_per_split, float* __restrict__ lat, float* __restrict__ part_acc,
+                                                               float* __restrict__ part_ml, int KS, int M) {
+  // the latent is padded with zeros to RP = 64 NBW components: every loop below has a compile-time trip count
+  constexpr int KT = 16, LDP = 20, LDS_S = 17, RP = 64 * NBW, LDC = RP + 4, DQ = RP / 4;
+  extern __shared__ float lds[];
+  const int row0 = blk_tab[2 * blockIdx.x], nrows = blk_tab[2 * blockIdx.x + 1];
+  const int nqv = nrows * H, qv0 = blockIdx.y * 16;
+  if (qv0 >= nqv) return;
+  float* Cl = lds;                       // [16 keys][LDC]
+  float* Ql = Cl + KT * LDC;             // [16 q][LDC]
+  float* Sp = Ql + 16 * LDC;             // [4 waves][16 q][LDS_S] partial scores
+  float* Pl = Sp + 4 * 16 * LDS_S;       // [16 q][LDP] weights
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c16 = lane & 15, g4 = lane >> 4;
+  const int64_t seq = row_seq[row0];
+  const int len_max = row_len[row0 + nrows - 1];
+  f32x4 v[NBW];
+  load16<NBW>(v, r, tid, [&](int q) { const int qv = min(qv0 + q, nqv - 1); return qabs + ((int64_t)(row0 + qv / H) * H + qv % H) * r; },
+              [&](int q) { return qv0 + q < nqv; });
+  store16<NBW, LDC>(Ql, v, tid);
+  int mylen[4];
+  float mrun[4], lrun[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int qv = qv0 + 4 * g4 + i;
+    mylen[i] = qv < nqv ? row_len[row0 + qv / H] : 0;
+    mrun[i] = -INFINITY;
+    lrun[i] = 0.f;
+  }
+  f32x4 acc[NBW];
+#pragma unroll
+  for (int b = 0; b < NBW; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int n_tiles = (len_max + KT - 1) / KT;
+  const int t0 = blockIdx.z * tiles_per_split, t1 = min(t0 + tiles_per_split, n_tiles);
+  const float* abase = arena + seq * t_max * r;
+  auto fetch = [&](int tile) {
+    const int k0 = tile * KT;
+    load16<NBW>(v, r, tid, [&](int j) { return abase + (int64_t)min(k0 + j, len_max - 1) * r; }, [&](int j) { return k0 + j < len_max; });
+  };
+  if (t0 < t1) fetch(t0);
+  for (int tile = t0; tile < t1; ++tile) {
+    const int key0 = tile * KT;
+    __syncthreads();                                             // the previous tile's latents and weights are consumed (first: Q is staged)
+    store16<NBW, LDC>(Cl, v, tid);
+    if (tile + 1 < t1) fetch(tile + 1);                          // in flight while this tile is multiplied
+    __syncthreads();
+    {                                                            // partial scores over this wave's quarter of the components
+      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+      const float* qa = Ql + c16 * LDC + wave * DQ + g4;
+      const float* cb = Cl + c16 * LDC + wave * DQ + g4;
+#pragma unroll
+      for (int it = 0; it < DQ / 4; ++it) s = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[4 * it], cb[4 * it], s, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) Sp[(wave * 16 + 4 * g4 + i) * LDS_S + c16] = s[i];
+    }
+    __syncthreads();
+    float p[4], corr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int o = (4 * g4 + i) * LDS_S + c16;
+      float sc = (Sp[o] + Sp[16 * LDS_S + o]) + (Sp[32 * LDS_S + o] + Sp[48 * LDS_S + o]);
+      if (key0 + c16 >= mylen[i]) sc = -INFINITY;
+      const float mnew = fmaxf(mrun[i], row16_max(sc));
+      p[i] = (sc == -INFINITY) ? 0.f : expf(sc - mnew);
+      corr[i] = (mrun[i] == -INFINITY) ? 0.f : expf(mrun[i] - mnew);
+      lrun[i] = lrun[i] * corr[i] + row16_sum(p[i]);
+      mrun[i] = mnew;
+      if (wave == 0) Pl[(4 * g4 + i) * LDP + c16] = p[i];
+    }
+#pragma unroll
+    for (int b = 0; b < NBW; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[b][i] *= corr[i];
+    __syncthreads();
+#pragma unroll
+    for (int k0 = 0; k0 < KT; k0 += 4) {
+      const float pa = Pl[c16 * LDP + k0 + g4];
+      const float* cb = Cl + (k0 + g4) * LDC + 16 * wave + c16;
+#pragma unroll
+      for (int b = 0; b < NBW; ++b) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa, cb[64 * b], acc[b], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int qv = qv0 + 4 * g4 + i;
+    if (qv >= nqv) continue;
+    const int64_t o = (int64_t)(row0 + qv / H) * H + qv % H;
+    const float inv = 1.0f / lrun[i];
+#pragma unroll
+    for (int b = 0; b < NBW; ++b) {
+      const int d = 16 * (wave + 4 * b) + c16;
+      if (d >= r) continue;
+      if (KS == 1) lat[o * r + d] = acc[b][i] * inv;
+      else part_acc[((int64_t)blockIdx.z * M * H + o) * r + d] = acc[b][i];
+    }
+    if (KS > 1 && wave == 0 && c16 == 0) {
+      const int64_t po = (int64_t)blockIdx.z * M * H + o;
+      part_ml[po * 2] = mrun[i];
+      part_ml[po * 2 + 1] = lrun[i];
+    }
+  }
+}
+
+// one wave per (row, head) and 64 latent components: combine the key splits (lane s holds split s's maximum and sum; KS <= 64)
 __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, int KS,
                                                            int MH, int r, float* __restrict__ lat) {
-  const int o = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int o = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, d = blockIdx.y * 64 + lane;
   if (o >= MH) return;
-  float mx = -INFINITY;
-  for (int s = 0; s < KS; ++s) mx = fmaxf(mx, part_ml[((int64_t)s * MH + o) * 2]);
-  float L = 0.f;
-  for (int s = 0; s < KS; ++s) {
-    const float ms = part_ml[((int64_t)s * MH + o) * 2];
-    if (ms != -INFINITY) L += expf(ms - mx) * part_ml[((int64_t)s * MH + o) * 2 + 1];
-  }
-  for (int d = lane; d < r; d += 64) {
-    float a = 0.f;
-    for (int s = 0; s < KS; ++s) {
-      const float ms = part_ml[((int64_t)s * MH + o) * 2];
-      if (ms != -INFINITY) a += expf(ms - mx) * part_acc[((int64_t)s * MH + o) * r + d];
-    }
-    lat[(int64_t)o * r + d] = a / L;
-  }
+  const float ms = lane < KS ? part_ml[((int64_t)lane * MH + o) * 2] : -INFINITY;
+  const float ls = lane < KS ? part_ml[((int64_t)lane * MH + o) * 2 + 1] : 0.f;
+  const float mx = wave_max(ms);
+  const float w = (ms == -INFINITY) ? 0.f : expf(ms - mx);
+  const float inv = 1.0f / wave_sum(w * ls);
+  const int dc = d < r ? d : r - 1;
+  float a = 0.f;
+#pragma unroll 16
+  for (int s = 0; s < KS; ++s) a = fmaf(lane_f(w, s), part_acc[((int64_t)s * MH + o) * r + dc], a);
+  if (d < r) lat[(int64_t)o * r + d] = a * inv;
 }
 
 }  // namespace
@@ -328,8 +589,10 @@ __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restri
 extern "C" int mn_affine_ln_rows(const float* x, int64_t ldx, const uint16_t* w, const uint16_t* b, float eps, float* y, int64_t ldy,
                                  uint16_t* y16, int64_t ldy16, int M, int n, void* stream) {
   MN_CHECK_ARG(x && w && b && (y || y16) && M >= 1 && n >= 1, "mn_affine_ln_rows: bad args");
-  hipLaunchKernelGGL(affine_ln_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), x, ldx, w, b, eps, y, ldy, y16, ldy16,
-                     M, n);
+  const RowArgs ra{x, ldx, nullptr, 0, nullptr, 0, w, b, eps, y, ldy, y16, ldy16, n};
+  if (!launch_row_block<ROW_LN>(ra, M, mn_stream(stream)))
+    hipLaunchKernelGGL(affine_ln_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), x, ldx, w, b, eps, y, ldy, y16, ldy16,
+                       M, n);
   MN_CHECK_LAUNCH("mn_affine_ln_rows");
   return MN_OK;
 }
@@ -337,8 +600,10 @@ extern "C" int mn_affine_ln_rows(const float* x, int64_t ldx, const uint16_t* w,
 extern "C" int mn_gated_ln_residual(float* x, int64_t ldx, const float* g, int64_t ldg, const float* y, int64_t ldy, const uint16_t* w,
                                     const uint16_t* b, float eps, int M, int n, void* stream) {
   MN_CHECK_ARG(x && g && y && w && b && M >= 1 && n >= 1, "mn_gated_ln_residual: bad args");
-  hipLaunchKernelGGL(gated_ln_residual_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), x, ldx, g, ldg, y, ldy, w, b,
-                     eps, M, n);
+  const RowArgs ra{nullptr, 0, g, ldg, y, ldy, w, b, eps, x, ldx, nullptr, 0, n};
+  if (!launch_row_block<ROW_GATED_LN_RESIDUAL>(ra, M, mn_stream(stream)))
+    hipLaunchKernelGGL(gated_ln_residual_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), x, ldx, g, ldg, y, ldy, w, b,
+                       eps, M, n);
   MN_CHECK_LAUNCH("mn_gated_ln_residual");
   return MN_OK;
 }
@@ -355,7 +620,9 @@ extern "C" int mn_rms_rows(const float* x, int64_t ldx, const uint16_t* w, float
 extern "C" int mn_polynorm_rows(const float* z, int64_t ldz, const uint16_t* coef, float eps, float* y, int64_t ldy, uint16_t* y16,
                                 int64_t ldy16, int M, int n, void* stream) {
   MN_CHECK_ARG(z && coef && (y || y16) && M >= 1 && n >= 1, "mn_polynorm_rows: bad args");
-  hipLaunchKernelGGL(polynorm_kernel, dim3((unsigned)M), dim3(256), 0, mn_stream(stream), z, ldz, coef, eps, y, ldy, y16, ldy16, n);
+  const RowArgs ra{z, ldz, nullptr, 0, nullptr, 0, coef, nullptr, eps, y, ldy, y16, ldy16, n};
+  if (!launch_row_block<ROW_POLYNORM>(ra, M, mn_stream(stream)))
+    hipLaunchKernelGGL(polynorm_kernel, dim3((unsigned)M), dim3(256), 0, mn_stream(stream), z, ldz, coef, eps, y, ldy, y16, ldy16, n);
   MN_CHECK_LAUNCH("mn_polynorm_rows");
   return MN_OK;
 }
@@ -396,7 +663,11 @@ extern "C" int mn_gemm_f32_batched(const float* A, int64_t lda, int64_t a_bs, co
   MN_CHECK_ARG(A && W && (C || C16) && M >= 1 && N >= 1 && K >= 1 && batch >= 1 && batch <= 65535, "mn_gemm_f32_batched: bad args");
   GemmF32 a{A, lda, a_bs, W, ldw, w_bs, bias, C, ldc, c_bs, C16, ldc16, c16_bs, G, ldg, g_bs, M, N, K, alpha};
   hipStream_t st = mn_stream(stream);
-  if (M <= 16) {
+  if (M <= 8) {
+    MN_CHECK_ARG(mn_cdiv(N, 4) <= 0x7fffffff, "mn_gemm_f32_batched: too many columns");
+    if (M <= 2) hipLaunchKernelGGL((gemv_f32_kernel<2>), dim3((unsigned)mn_cdiv(N, 4), 1, (unsigned)batch), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemv_f32_kernel<8>), dim3((unsigned)mn_cdiv(N, 4), 1, (unsigned)batch), dim3(256), 0, st, a);
+  } else if (M <= 16) {
     hipLaunchKernelGGL((gemm_f32_kernel<1>), dim3((unsigned)mn_cdiv(N, 64), 1, (unsigned)batch), dim3(256), 0, st, a);
   } else {
     MN_CHECK_ARG(mn_cdiv(M, 64) <= 65535, "mn_gemm_f32_batched: too many rows");
@@ -408,15 +679,15 @@ extern "C" int mn_gemm_f32_batched(const float* A, int64_t lda, int64_t a_bs, co
 
 // rows of a workgroup (consecutive rows of one sequence) and the key-tile length for latent size r
 extern "C" int mn_latent_attn_block_rows(void) { return 4; }
-static inline int latent_kt(int r) { return r <= 256 ? 64 : r <= 512 ? 32 : 16; }   // the tile [KT][r + 1] fp32 stays below 66 KiB
+static inline int latent_kt(int r, int variant) { return variant == MN_LATENT_ATTN_VALU ? (r <= 256 ? 64 : r <= 512 ? 32 : 16) : 16; }   // VALU: the tile [KT][r + 1] fp32 stays below 66 KiB
 
 extern "C" int mn_latent_attn_splits(int n_blk, int max_len, int r) {
-  const int KT = latent_kt(r);
-  const int tiles = (int)mn_cdiv(max_len > 0 ? max_len : 1, KT);
+  const int tiles = (int)mn_cdiv(max_len > 0 ? max_len : 1, 16);
   int ks = (int)mn_cdiv(2 * (int64_t)mn_num_cus(), n_blk > 0 ? n_blk : 1);
-  const int cap = (int)mn_cdiv(tiles, 2);              // a split works on at least 2 key tiles
+  const int cap = (int)mn_cdiv(tiles, 4);              // a split works on at least 64 keys
   if (ks > cap) ks = cap;
   if (ks > 64) ks = 64;
+  (void)r;
   return ks < 1 ? 1 : ks;
 }
 
@@ -424,23 +695,47 @@ extern "C" size_t mn_latent_attn_workspace_bytes(int M, int H, int r, int ks) {
   return ks <= 1 ? 0 : (size_t)ks * M * H * (r + 2) * sizeof(float);
 }
 
-extern "C" int mn_latent_attn(const float* qabs, const float* arena, const int32_t* row_seq, const int32_t* row_len, const int32_t* blk_tab,
-                              int n_blk, int M, int H, int r, int t_max, int max_len, int ks, float* lat, void* ws, size_t ws_bytes,
-                              void* stream) {
+extern "C" int mn_latent_attn_ex(const float* qabs, const float* arena, const int32_t* row_seq, const int32_t* row_len,
+                                 const int32_t* blk_tab, int n_blk, int M, int H, int r, int t_max, int max_len, int ks, float* lat, void* ws,
+                                 size_t ws_bytes, int variant, void* stream) {
   MN_CHECK_ARG(qabs && arena && row_seq && row_len && blk_tab && lat && n_blk >= 1 && M >= 1 && H >= 1 && r >= 1 && t_max >= 1,
                "mn_latent_attn: bad args");
   MN_CHECK_ARG(r <= 1024, "mn_latent_attn: latent size %d above 1024 is not supported", r);
-  MN_CHECK_ARG(max_len >= 1 && max_len <= t_max && ks >= 1 && ks <= 65535, "mn_latent_attn: bad max_len=%d / ks=%d", max_len, ks);
+  MN_CHECK_ARG(max_len >= 1 && max_len <= t_max && ks >= 1 && ks <= 64, "mn_latent_attn: bad max_len=%d / ks=%d (1 .. 64 key splits)", max_len, ks);
   MN_CHECK_ARG(ws_bytes >= mn_latent_attn_workspace_bytes(M, H, r, ks) && (ks == 1 || ws), "mn_latent_attn: workspace too small");
-  const int KT = latent_kt(r), RB = mn_latent_attn_block_rows();
+  MN_CHECK_ARG(variant == MN_LATENT_ATTN_MFMA || variant == MN_LATENT_ATTN_VALU, "mn_latent_attn: unknown variant %d", variant);
+  const int KT = latent_kt(r, variant), RB = mn_latent_attn_block_rows();
   const int tiles = (int)mn_cdiv(max_len, KT), tps = (int)mn_cdiv(tiles, ks);
-  const int nw = RB * H < 16 ? RB * H : 16;
-  const dim3 grid((unsigned)n_blk, (unsigned)mn_cdiv(RB * H, nw), (unsigned)ks), block((unsigned)(64 * nw));
-  MN_CHECK_ARG(grid.y <= 65535, "mn_latent_attn: too many heads");
-  const size_t lds = (size_t)KT * (r + 1) * sizeof(float);
   float* pacc = reinterpret_cast<float*>(ws);
   float* pml = pacc ? pacc + (size_t)ks * M * H * r : nullptr;
   hipStream_t st = mn_stream(stream);
+  if (variant == MN_LATENT_ATTN_MFMA) {
+    const int nbw = (int)mn_cdiv(r, 64);
+    const int inst = nbw <= 4 ? nbw : nbw <= 6 ? 6 : nbw <= 8 ? 8 : nbw <= 12 ? 12 : 16;      // instantiated paddings: 64 .. 256, 384, 512, 768, 1024
+    const size_t lds = ((size_t)32 * (64 * inst + 4) + 4 * 16 * 17 + 16 * 20) * sizeof(float);
+    const dim3 grid((unsigned)n_blk, (unsigned)mn_cdiv(RB * H, 16), (unsigned)ks);
+    MN_CHECK_ARG(grid.y <= 65535 && ks <= 64, "mn_latent_attn: too many heads or key splits");
+#define MN_LM(N_)                                                                                                                   \
+  do {                                                                                                                              \
+    static bool attr_set = false;                                                                                                   \
+    if (!attr_set) {                                                                                                                \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(latent_attn_mfma_kernel<N_>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                144 * 1024);                                                                                        \
+      attr_set = true;                                                                                                              \
+    }                                                                                                                               \
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<N_>), grid, dim3(256), lds, st, qabs, arena, row_seq, row_len, blk_tab, H, r, t_max, tps, \
+                       lat, pacc, pml, ks, M);                                                                                      \
+  } while (0)
+    switch (inst) {
+      case 1: MN_LM(1); break; case 2: MN_LM(2); break; case 3: MN_LM(3); break; case 4: MN_LM(4); break;
+      case 6: MN_LM(6); break; case 8: MN_LM(8); break; case 12: MN_LM(12); break; default: MN_LM(16); break;
+    }
+#undef MN_LM
+  } else {
+    const int nw = RB * H < 16 ? RB * H : 16;
+    const dim3 grid((unsigned)n_blk, (unsigned)mn_cdiv(RB * H, nw), (unsigned)ks), block((unsigned)(64 * nw));
+    MN_CHECK_ARG(grid.y <= 65535, "mn_latent_attn: too many heads");
+    const size_t lds = (size_t)KT * (r + 1) * sizeof(float);
 #define MN_LA(R_)                                                                                                                   \
   do {                                                                                                                              \
     static bool attr_set = false;                                                                                                   \
@@ -451,12 +746,21 @@ extern "C" int mn_latent_attn(const float* qabs, const float* arena, const int32
     hipLaunchKernelGGL((latent_attn_kernel<R_>), grid, block, lds, st, qabs, arena, row_seq, row_len, blk_tab, H, r, t_max, KT, tps, lat, \
                        pacc, pml, ks, M);                                                                                           \
   } while (0)
-  if (r <= 64) MN_LA(1); else if (r <= 128) MN_LA(2); else if (r <= 256) MN_LA(4); else if (r <= 512) MN_LA(8); else MN_LA(16);
+    if (r <= 64) MN_LA(1); else if (r <= 128) MN_LA(2); else if (r <= 256) MN_LA(4); else if (r <= 512) MN_LA(8); else MN_LA(16);
 #undef MN_LA
+  }
   MN_CHECK_LAUNCH("mn_latent_attn");
   if (ks > 1) {
-    hipLaunchKernelGGL(latent_merge_kernel, dim3((unsigned)mn_cdiv((int64_t)M * H, 4)), dim3(256), 0, st, pacc, pml, ks, M * H, r, lat);
+    hipLaunchKernelGGL(latent_merge_kernel, dim3((unsigned)mn_cdiv((int64_t)M * H, 4), (unsigned)mn_cdiv(r, 64)), dim3(256), 0, st, pacc, pml, ks, M * H, r,
+                       lat);
     MN_CHECK_LAUNCH("mn_latent_attn(merge)");
   }
   return MN_OK;
+}
+
+extern "C" int mn_latent_attn(const float* qabs, const float* arena, const int32_t* row_seq, const int32_t* row_len, const int32_t* blk_tab,
+                              int n_blk, int M, int H, int r, int t_max, int max_len, int ks, float* lat, void* ws, size_t ws_bytes,
+                              void* stream) {
+  return mn_latent_attn_ex(qabs, arena, row_seq, row_len, blk_tab, n_blk, M, H, r, t_max, max_len, ks, lat, ws, ws_bytes,
+                           MN_LATENT_ATTN_MFMA, stream);
 }

@@ -76,6 +76,16 @@ def run_pizitar(s, T, batches, n_dec):
                 dec.step(xb, row_seq, slot, back, ln, blk, T + i + 1)
                 check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
         out[f"decode_b{B}_tokens_per_s"] = B * n_dec / _time(loop, 2, 1)
+        slot_g = torch.full((B,), T, dtype=torch.int32, device=dev)
+        ln_g = slot_g + 1
+        graph = dec.decode_graph(row_seq, slot_g, ln_g)
+
+        def loop_graph():
+            slot_g.fill_(T)
+            ln_g.fill_(T + 1)
+            for i in range(n_dec):
+                graph.run(xb, T + i + 1)
+        out[f"decode_b{B}_graph_tokens_per_s"] = B * n_dec / _time(loop_graph, 2, 1)
     # the attention kernel alone
     H, r = s["heads"], s["kv_rank"]
     tabs = {k: (torch.from_numpy(v).to(dev) if k != "max_len" else v) for k, v in

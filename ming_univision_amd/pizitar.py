@@ -184,7 +184,7 @@ class PizitarDecoder:
             self._ws[key] = torch.empty(need, dtype=torch.uint8, device=self.device)
         return self._ws[key]
 
-    def step(self, x, row_seq, row_slot, row_back, row_len, blk_tab, max_len, out=None, trace=None):
+    def step(self, x, row_seq, row_slot, row_back, row_len, blk_tab, max_len, out=None, trace=None, ws=None):
         """One pass of the stack over M rows.  x fp32 [M, width] (input embeddings); int32 device arrays per row (row r is
         position row_slot[r] of cache sequence row_seq[r], preceded in this pass by row_back[r] rows of its sequence, and attends
         row_len[r] = row_slot[r] + 1 slots); blk_tab int32 [n_blk, 2] cuts the rows into runs of <= block_rows consecutive rows of
@@ -201,7 +201,8 @@ class PizitarDecoder:
             out = torch.empty(M, self.cfg.width, dtype=torch.float32, device=self.device)
         if trace is not None:
             assert trace.dtype == torch.float32 and trace.is_contiguous() and tuple(trace.shape) == (len(self.cfg.layers), M, self.cfg.width)
-        ws = self._workspace(M, max_len)
+        if ws is None:
+            ws = self._workspace(M, max_len)
         check(lib().mn_seq_step(C.byref(self.struct), C.byref(self.state), ptr(x), x.stride(0), M, ptr(row_seq), ptr(row_slot),
                                 ptr(row_back), ptr(row_len), ptr(blk_tab), blk_tab.shape[0], int(max_len), ptr(out), ptr(trace),
                                 ptr(ws), ws.numel(), current_stream()), "mn_seq_step")
@@ -242,6 +243,10 @@ class PizitarDecoder:
                                     torch.stack([torch.arange(B, dtype=torch.int32), torch.ones(B, dtype=torch.int32)], 1).contiguous().to(self.device))
         return self._decode_tabs[B]
 
+    def decode_graph(self, row_seq, row_slot, row_len):
+        """A replayable lock-step decode step of B = len(row_seq) sequences (one row each): `DecodeGraph`."""
+        return DecodeGraph(self, row_seq, row_slot, row_len)
+
     # ---- vocabulary -------------------------------------------------------------------------------------------------------------
     def embed(self, ids):
         return ops.bf16_to_f32(self.embed_w[ids.reshape(-1).to(self.device)])
@@ -270,6 +275,48 @@ class PizitarDecoder:
         return ops.sample_logits(self.logits(hidden), u, temperature, top_k, top_p)
 
 
+class DecodeGraph:
+    """One lock-step decode step (stack pass + advancing the rows' slots and lengths) captured as a HIP graph: a step of a small
+    model is some twenty short launches per layer, and their host-side launch cost, not the kernels, bounds it.  The per-row
+    state lives in device arrays that the graph's own last node advances, the input rows are copied into a fixed buffer, and the
+    only host number baked in is an upper bound of the lengths (it sizes the attention's key splits), so one capture serves
+    `span` tokens; `run` re-captures when the lengths pass the bound."""
+
+    def __init__(self, dec, row_seq, row_slot, row_len, span=256):
+        self.dec, self.span = dec, span
+        self.row_seq, self.slot, self.len = row_seq, row_slot, row_len
+        B = row_seq.numel()
+        self.B = B
+        self.back, self.blk = dec.decode_tables(B)
+        self.x = torch.zeros(B, dec.cfg.width, dtype=torch.float32, device=dec.device)
+        self.out = torch.empty(B, dec.cfg.width, dtype=torch.float32, device=dec.device)
+        n = int(lib().mn_seq_workspace_bytes(C.byref(dec.struct), B, dec.t_max))
+        self.ws = torch.empty(n, dtype=torch.uint8, device=dec.device)
+        self.bound, self.graph = 0, None
+
+    def _body(self):
+        self.dec.step(self.x, self.row_seq, self.slot, self.back, self.len, self.blk, self.bound, out=self.out, ws=self.ws)
+        check(lib().mn_rows_advance(ptr(self.slot), ptr(self.len), None, self.B, 1, current_stream()), "mn_rows_advance")
+
+    def run(self, x, max_len):
+        """x fp32 [B, width]: the new tokens' embeddings; max_len: host upper bound of the lengths after this step.
+        Returns the hidden states [B, width] (a fixed buffer, overwritten by the next run)."""
+        if self.graph is None or max_len > self.bound:
+            self.bound = min(self.dec.t_max, (max_len + self.span - 1) // self.span * self.span)
+            self.graph = torch.cuda.CUDAGraph()
+            self.x.copy_(x)
+            torch.cuda.synchronize(self.dec.device)
+            snap = (self.slot.clone(), self.len.clone())
+            with torch.cuda.graph(self.graph):
+                self._body()
+            # capture records, it does not run: the arrays are untouched, but restore them in case a runtime ever executes eagerly
+            self.slot.copy_(snap[0])
+            self.len.copy_(snap[1])
+        self.x.copy_(x)
+        self.graph.replay()
+        return self.out
+
+
 class PizitarForCausalLM:
     """Generation entry point: requests in, token ids out, in lock-step batches (the batching of the other decoder's
     `generate_text_batch`): all prompts share the prefill passes, then one pass per new token serves every live sequence."""
@@ -284,9 +331,11 @@ class PizitarForCausalLM:
         return cls(PizitarDecoder.from_pretrained(path, device=device, t_max=t_max, arith=arith), eos_token_id)
 
     @torch.no_grad()
-    def generate(self, prompts, max_new_tokens=16, do_sample=False, temperature=1.0, top_k=50, top_p=1.0, generator=None, sync_every=8):
+    def generate(self, prompts, max_new_tokens=16, do_sample=False, temperature=1.0, top_k=50, top_p=1.0, generator=None, sync_every=8,
+                 use_graph=None):
         """prompts: list of token-id lists (unequal lengths allowed).  Greedy, or sampled (new token i of request b uses uniform
-        [i, b] of one torch.rand(max_new_tokens, B) draw).  Returns the new tokens of every request (cut after the first EOS)."""
+        [i, b] of one torch.rand(max_new_tokens, B) draw).  use_graph: run the decode steps as replays of a captured HIP graph
+        (default: from 8 new tokens on).  Returns the new tokens of every request (cut after the first EOS)."""
         dec, dev = self.dec, self.dec.device
         B = len(prompts)
         lens = [len(p) for p in prompts]
@@ -302,6 +351,7 @@ class PizitarForCausalLM:
             slot = torch.tensor(lens, dtype=torch.int32, device=dev)
             ln = slot + 1
             back, blk = dec.decode_tables(B)
+            graph = dec.decode_graph(row_seq, slot, ln) if (max_new_tokens >= 8 if use_graph is None else use_graph) else None
             finished = torch.zeros(B, dtype=torch.bool, device=dev)
             uniforms = torch.rand(max_new_tokens, B, device=dev, generator=generator) if do_sample else None
             toks = []
@@ -314,8 +364,11 @@ class PizitarForCausalLM:
                         break
                 if i + 1 == max_new_tokens:
                     break
-                hidden = dec.step(dec.embed(tok), row_seq, slot, back, ln, blk, max(lens) + i + 1)
-                check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
+                if graph is not None:
+                    hidden = graph.run(dec.embed(tok), max(lens) + i + 1)
+                else:
+                    hidden = dec.step(dec.embed(tok), row_seq, slot, back, ln, blk, max(lens) + i + 1)
+                    check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
             out = torch.stack(toks, 1).tolist()
         finally:
             for s in seqs:

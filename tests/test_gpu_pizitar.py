@@ -153,8 +153,11 @@ def test_fp32_batched_product():
         assert err(c, ref) < 1e-5 and err(c16.float(), ref) < 1e-2
 
 
-def _attend(q, arena, seq, lens, H, r, block_rows, ks):
-    """mn_latent_attn on rows that are consecutive positions of ONE sequence."""
+VARIANTS = {"mfma": 0, "valu": 1}
+
+
+def _attend(q, arena, seq, lens, H, r, block_rows, ks, variant="mfma"):
+    """mn_latent_attn_ex (fp32 matrix-core kernel or the plain one) on rows that are consecutive positions of ONE sequence."""
     from ming_univision_amd._lib import check, current_stream, lib, ptr
     M = q.shape[0]
     row_seq = torch.full((M,), seq, dtype=torch.int32, device="cuda")
@@ -164,15 +167,16 @@ def _attend(q, arena, seq, lens, H, r, block_rows, ks):
     lat = torch.empty(M, H, r, device="cuda")
     nb = lib().mn_latent_attn_workspace_bytes(M, H, r, ks)
     ws = torch.empty(max(nb, 16), dtype=torch.uint8, device="cuda")
-    check(lib().mn_latent_attn(ptr(q), ptr(arena), ptr(row_seq), ptr(row_len), ptr(blk), blk.shape[0], M, H, r, arena.shape[1], max(lens), ks,
-                               ptr(lat), ptr(ws), ws.numel(), current_stream()))
+    check(lib().mn_latent_attn_ex(ptr(q), ptr(arena), ptr(row_seq), ptr(row_len), ptr(blk), blk.shape[0], M, H, r, arena.shape[1], max(lens), ks,
+                                  ptr(lat), ptr(ws), ws.numel(), VARIANTS[variant], current_stream()))
     return lat
 
 
-@pytest.mark.parametrize("r,H", [(40, 3), (64, 4), (72, 1), (136, 2), (264, 2), (520, 1)])
-def test_latent_attention_needles(r, H):
+@pytest.mark.parametrize("variant", list(VARIANTS))
+@pytest.mark.parametrize("r,H", [(40, 3), (64, 4), (72, 1), (136, 2), (264, 2), (520, 1), (64, 20)])
+def test_latent_attention_needles(r, H, variant):
     """One key is made to dominate (the query is a large multiple of that key's latent): the result is that latent if and only if
-    the key is inside the row's length.  Needles at the first slot, around the kernel's key-tile edges (32 / 64 keys), around the
+    the key is inside the row's length.  Needles at the first slot, around the kernel's key-tile edges (16 / 32 / 64 keys), around the
     edges of forced key splits, and at the row's last visible slot; the same query with the length one shorter must not see it."""
     from ming_univision_amd._lib import lib
     g = torch.Generator().manual_seed(r)
@@ -180,11 +184,11 @@ def test_latent_attention_needles(r, H):
     arena = torch.randn(2, T, r, generator=g)
     ad = arena.cuda()
     for ks in (1, 3):
-        for needle in (0, 1, 31, 32, 33, 63, 64, 65, 127, 128, 191, 192, 255, 256, 298, 299):
+        for needle in (0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 95, 96, 127, 128, 191, 192, 255, 256, 298, 299):
             c = arena[1, needle].double()
             q1 = (40.0 / float(c @ c)) * c                                  # score 40 at the needle, |score| ~ 40 / sqrt(r) elsewhere
             q = torch.stack([torch.stack([q1.float() * (1 + 0.01 * h) for h in range(H)])] * 2)         # two rows, same query
-            lat = _attend(q.cuda(), ad, 1, [needle, needle + 1] if needle else [1, 1], H, r, br, ks)
+            lat = _attend(q.cuda(), ad, 1, [needle, needle + 1] if needle else [1, 1], H, r, br, ks, variant)
             ref = []
             for ln in ([needle, needle + 1] if needle else [1, 1]):
                 p = torch.softmax(arena[1, :ln].double() @ q[0].double().T, 0)                         # [ln, H]
@@ -196,7 +200,8 @@ def test_latent_attention_needles(r, H):
                 assert float((lat[0, 0].cpu().double() - c).abs().max()) > 0.1 * float(c.abs().max()), (ks, needle)
 
 
-def test_latent_attention_against_expanded_heads():
+@pytest.mark.parametrize("variant", list(VARIANTS))
+def test_latent_attention_against_expanded_heads(variant):
     """Absorbed attention (queries mapped into latent space, values expanded afterwards) = attention on per-head keys and values."""
     g = torch.Generator().manual_seed(5)
     H, d, v, r, T = 3, 24, 16, 40, 150
@@ -208,7 +213,7 @@ def test_latent_attention_against_expanded_heads():
     arena = torch.zeros(1, T + 5, r)
     arena[0, :T] = c
     for block_rows, ks in ((4, 1), (1, 2), (3, 4)):
-        lat = _attend(qabs.cuda(), arena.cuda(), 0, list(range(1, T + 1)), H, r, block_rows, ks).cpu().double()
+        lat = _attend(qabs.cuda(), arena.cuda(), 0, list(range(1, T + 1)), H, r, block_rows, ks, variant).cpu().double()
         out = torch.cat([lat[:, h] @ uv[h * v:(h + 1) * v].double().T for h in range(H)], 1)
         assert err(out, ref) < 1e-5
 
@@ -337,6 +342,36 @@ def test_greedy_generation_entry_point():
     assert not lm.slots.length and lm.slots.next == 3
     out = lm.generate(prompts, max_new_tokens=5, do_sample=True, top_k=8, generator=torch.Generator(device="cuda").manual_seed(0))
     assert all(len(o) == 5 and all(0 <= x < cfg["vocab"] for x in o) for o in out) and not lm.slots.length
+
+
+def test_decode_graph_replays():
+    """The captured decode step against the eager one: every replay is checked (not only the first), with eager work and host
+    synchronisations between replays, across a re-capture (the lengths pass the captured bound) and the 16-key tile edges."""
+    cfg, sd, dec = make("mixed", n_seq=3)
+    prompts = {0: toks(cfg, 21, 1), 1: toks(cfg, 5, 2), 2: toks(cfg, 40, 3)}
+    follow = {s: toks(cfg, 30, 10 + s) for s in prompts}
+    refs = {s: O.logits_of(cfg, sd, prompts[s] + follow[s]) for s in prompts}
+    for s, p in prompts.items():
+        run_portions(dec, s, p, [len(p)])
+    row_seq = torch.tensor(list(prompts), dtype=torch.int32, device="cuda")
+    slot = torch.tensor([len(p) for p in prompts.values()], dtype=torch.int32, device="cuda")
+    ln = slot + 1
+    g = dec.decode_graph(row_seq, slot, ln)
+    g.span = 16                                               # re-capture every 16 tokens
+    other = dec.embed(torch.tensor(toks(cfg, 7, 99), device="cuda"))
+    for i in range(30):
+        ids = torch.tensor([follow[s][i] for s in prompts], device="cuda")
+        hid = g.run(dec.embed(ids), max(len(p) for p in prompts.values()) + i + 1)
+        lg = dec.logits(hid.clone())
+        torch.cuda.synchronize()
+        for k, s in enumerate(prompts):
+            assert err(lg[k:k + 1], refs[s][len(prompts[s]) + i][None]) < 1e-4, (i, s)
+        dec.logits(other)                                     # eager work between replays
+    assert slot.tolist() == [len(p) + 30 for p in prompts.values()]
+    from ming_univision_amd.pizitar import PizitarForCausalLM
+    lm = PizitarForCausalLM(dec)
+    ps = [toks(cfg, 9, 5), toks(cfg, 30, 6)]
+    assert lm.generate(ps, max_new_tokens=20, use_graph=True) == lm.generate(ps, max_new_tokens=20, use_graph=False)
 
 
 def test_trace_runner(tmp_path):
