@@ -420,8 +420,9 @@ __global__ __launch_bounds__(1024) void latent_attn_kernel(const float* __restri
 // Latent attention on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: fp32 operands, fp32 accumulate — scores and weights stay
 // 32-bit).  A workgroup of 4 waves owns 16 query vectors (row, head) of one run of rows and walks the sequence's latents in tiles
 // of 16 keys staged in LDS:
-//   scores   S[16 q, 16 keys] = Q C^T: every wave multiplies its quarter of the latent components, the partial tiles are summed
-//            through LDS, so all four waves hold the same scores and keep the same running maximum / sum without talking
+//   scores   S[16 q, 16 keys] = Q C^T: every wave multiplies its quarter of the latent components (its slice of Q stays in
+//            registers), the partial tiles are summed through LDS, so all four waves hold the same scores and keep the same
+//            running maximum / sum without talking
 //   values   O[16 q, r] += P C: the weights go through LDS into the A-operand layout, wave w owns the 16-column blocks w, w + 4, ..
 // Operand layouts (lane l, c = l % 16, g = l / 16): A[row c][k g], B[k g][col c], D[row 4 g + i][col c] in VGPR i.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -473,16 +474,24 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
   const int nqv = nrows * H, qv0 = blockIdx.y * 16;
   if (qv0 >= nqv) return;
   float* Cl = lds;                       // [16 keys][LDC]
-  float* Ql = Cl + KT * LDC;             // [16 q][LDC]
-  float* Sp = Ql + 16 * LDC;             // [4 waves][16 q][LDS_S] partial scores
+  float* Sp = Cl + KT * LDC;             // [4 waves][16 q][LDS_S] partial scores
   float* Pl = Sp + 4 * 16 * LDS_S;       // [16 q][LDP] weights
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c16 = lane & 15, g4 = lane >> 4;
   const int64_t seq = row_seq[row0];
   const int len_max = row_len[row0 + nrows - 1];
   f32x4 v[NBW];
-  load16<NBW>(v, r, tid, [&](int q) { const int qv = min(qv0 + q, nqv - 1); return qabs + ((int64_t)(row0 + qv / H) * H + qv % H) * r; },
-              [&](int q) { return qv0 + q < nqv; });
-  store16<NBW, LDC>(Ql, v, tid);
+  // the A operands of this wave's score products stay in registers for the whole key walk: query c16, components wave DQ + 4 it + g4
+  float qreg[DQ / 4];
+  {
+    const int qv = min(qv0 + c16, nqv - 1);
+    const float* src = qabs + ((int64_t)(row0 + qv / H) * H + qv % H) * r;
+#pragma unroll
+    for (int it = 0; it < DQ / 4; ++it) {
+      const int d = wave * DQ + 4 * it + g4;
+      const float t = src[d < r ? d : 0];
+      qreg[it] = (qv0 + c16 < nqv && d < r) ? t : 0.f;
+    }
+  }
   int mylen[4];
   float mrun[4], lrun[4];
 #pragma unroll
@@ -505,16 +514,15 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
   if (t0 < t1) fetch(t0);
   for (int tile = t0; tile < t1; ++tile) {
     const int key0 = tile * KT;
-    __syncthreads();                                             // the previous tile's latents and weights are consumed (first: Q is staged)
+    __syncthreads();                                             // the previous tile's latents and weights are consumed
     store16<NBW, LDC>(Cl, v, tid);
     if (tile + 1 < t1) fetch(tile + 1);                          // in flight while this tile is multiplied
     __syncthreads();
     {                                                            // partial scores over this wave's quarter of the components
       f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
-      const float* qa = Ql + c16 * LDC + wave * DQ + g4;
       const float* cb = Cl + c16 * LDC + wave * DQ + g4;
 #pragma unroll
-      for (int it = 0; it < DQ / 4; ++it) s = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[4 * it], cb[4 * it], s, 0, 0, 0);
+      for (int it = 0; it < DQ / 4; ++it) s = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[it], cb[4 * it], s, 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < 4; ++i) Sp[(wave * 16 + 4 * g4 + i) * LDS_S + c16] = s[i];
     }
@@ -712,7 +720,7 @@ extern "C" int mn_latent_attn_ex(const float* qabs, const float* arena, const in
   if (variant == MN_LATENT_ATTN_MFMA) {
     const int nbw = (int)mn_cdiv(r, 64);
     const int inst = nbw <= 4 ? nbw : nbw <= 6 ? 6 : nbw <= 8 ? 8 : nbw <= 12 ? 12 : 16;      // instantiated paddings: 64 .. 256, 384, 512, 768, 1024
-    const size_t lds = ((size_t)32 * (64 * inst + 4) + 4 * 16 * 17 + 16 * 20) * sizeof(float);
+    const size_t lds = ((size_t)16 * (64 * inst + 4) + 4 * 16 * 17 + 16 * 20) * sizeof(float);
     const dim3 grid((unsigned)n_blk, (unsigned)mn_cdiv(RB * H, 16), (unsigned)ks);
     MN_CHECK_ARG(grid.y <= 65535 && ks <= 64, "mn_latent_attn: too many heads or key splits");
 #define MN_LM(N_)                                                                                                                   \
