@@ -461,6 +461,17 @@ __device__ __forceinline__ void store16(float* __restrict__ dst, const f32x4 (&v
   for (int ps = 0; ps < NBW; ++ps) *reinterpret_cast<f32x4*>(dst + j * LDC + 4 * (cg + 16 * ps)) = v[ps];
 }
 
+// Workgroup barrier that orders LDS traffic only: the compiler's __syncthreads also drains the global loads in flight, which would
+// put the prefetched tile's memory latency back on every barrier of the key walk.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+}
+
+// exp on the hardware's base-2 exponential (one multiply + v_exp_f32, about 1e-6 relative over the softmax's range): the library
+// expf is some forty instructions, and eight of them per 16-key tile in every wave were the larger part of the key walk's time
+__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
+
 template <int NBW>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __restrict__ qabs, const float* __restrict__ arena,
                                                                const int32_t* __restrict__ row_seq, const int32_t* __restrict__ row_len,
@@ -514,19 +525,23 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
   if (t0 < t1) fetch(t0);
   for (int tile = t0; tile < t1; ++tile) {
     const int key0 = tile * KT;
-    __syncthreads();                                             // the previous tile's latents and weights are consumed
+    lds_barrier();                                             // the previous tile's latents and weights are consumed
     store16<NBW, LDC>(Cl, v, tid);
     if (tile + 1 < t1) fetch(tile + 1);                          // in flight while this tile is multiplied
-    __syncthreads();
+    lds_barrier();
     {                                                            // partial scores over this wave's quarter of the components
-      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f}, s2 = f32x4{0.f, 0.f, 0.f, 0.f};      // two chains: a product does not wait for the one before it
       const float* cb = Cl + c16 * LDC + wave * DQ + g4;
 #pragma unroll
-      for (int it = 0; it < DQ / 4; ++it) s = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[it], cb[4 * it], s, 0, 0, 0);
+      for (int it = 0; it < DQ / 4; it += 2) {
+        s = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[it], cb[4 * it], s, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[it + 1], cb[4 * it + 4], s2, 0, 0, 0);
+      }
+      s += s2;
 #pragma unroll
       for (int i = 0; i < 4; ++i) Sp[(wave * 16 + 4 * g4 + i) * LDS_S + c16] = s[i];
     }
-    __syncthreads();
+    lds_barrier();
     float p[4], corr[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -534,8 +549,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
       float sc = (Sp[o] + Sp[16 * LDS_S + o]) + (Sp[32 * LDS_S + o] + Sp[48 * LDS_S + o]);
       if (key0 + c16 >= mylen[i]) sc = -INFINITY;
       const float mnew = fmaxf(mrun[i], row16_max(sc));
-      p[i] = (sc == -INFINITY) ? 0.f : expf(sc - mnew);
-      corr[i] = (mrun[i] == -INFINITY) ? 0.f : expf(mrun[i] - mnew);
+      p[i] = (sc == -INFINITY) ? 0.f : fast_exp(sc - mnew);
+      corr[i] = (mrun[i] == -INFINITY) ? 0.f : fast_exp(mrun[i] - mnew);
       lrun[i] = lrun[i] * corr[i] + row16_sum(p[i]);
       mrun[i] = mnew;
       if (wave == 0) Pl[(4 * g4 + i) * LDP + c16] = p[i];
@@ -544,11 +559,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(const float* __re
     for (int b = 0; b < NBW; ++b)
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[b][i] *= corr[i];
-    __syncthreads();
+    lds_barrier();
+    // step t multiplies keys t, t + 4, t + 8, t + 12 (lane group g4 holds key t + 4 g4): with the row stride 4 mod 32 their rows
+    // start 16 banks apart pairwise, so the 64 lanes' reads spread two per bank — consecutive keys would pile four on some
 #pragma unroll
-    for (int k0 = 0; k0 < KT; k0 += 4) {
-      const float pa = Pl[c16 * LDP + k0 + g4];
-      const float* cb = Cl + (k0 + g4) * LDC + 16 * wave + c16;
+    for (int t = 0; t < 4; ++t) {
+      const float pa = Pl[c16 * LDP + t + 4 * g4];
+      const float* cb = Cl + (t + 4 * g4) * LDC + 16 * wave + c16;
 #pragma unroll
       for (int b = 0; b < NBW; ++b) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa, cb[64 * b], acc[b], 0, 0, 0);
     }

@@ -272,6 +272,24 @@ def test_unequal_requests_share_a_pass():
     assert err(lg[0:1], refs[0][8:9]) < 1e-4 and err(lg[1:31], refs[3][40:70]) < 1e-4 and err(lg[31:32], refs[2][32:33]) < 1e-4
 
 
+def test_inputs_longer_than_a_pass(monkeypatch):
+    """More rows than one pass through the stack takes: the passes cut a sequence in the middle (inside the filter's reach and
+    inside a key tile) and a later sequence starts inside a pass; the per-layer trace is stitched across passes."""
+    from ming_univision_amd import pizitar
+    monkeypatch.setattr(pizitar, "MAX_ROWS", 37)
+    cfg, sd, dec = make("mixed", n_seq=2)
+    a, b = toks(cfg, 90, 1), toks(cfg, 50, 2)
+    trace = []
+    ra, rb = O.logits_of(cfg, sd, a, trace=trace), O.logits_of(cfg, sd, b)
+    ids = torch.tensor(a + b, device="cuda")
+    hid, tr = dec.forward_spans(dec.embed(ids), [(1, 90, 0), (0, 50, 0)], trace=True)
+    lg = dec.logits(hid)
+    assert err(lg[:90], ra) < 1e-4 and err(lg[90:], rb) < 1e-4
+    assert err(tr[-1][:90], trace[-1]) < 1e-4
+    with pytest.raises(AssertionError):
+        dec.forward_spans(dec.embed(ids[:10]), [(0, 10, dec.t_max - 5)])       # beyond the arena: refused, not written
+
+
 def test_released_sequences_are_reused():
     """A cache sequence that held a longer request is given back and reused: the old latents and filter state stay in memory and
     must not leak into the next request (nothing is cleared; lengths bound every read)."""
