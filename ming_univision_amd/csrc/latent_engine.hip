@@ -1,7 +1,8 @@
 // latent_engine.hip — the step function of latent-cache sequence models (mingnative.h section 9): one pass of the layer stack
 // over the rows of a step as a chain of launches on the caller's stream.  Matrix products are routed per call:
 //   M <= 8 rows                      mn_skinny_gemm (weight streaming, fp32 FMA) — the decode route of the other decoder too
-//   MN_SEQ_ARITH_BF16, M > 8         mn_gemm_bf16 on the bf16 copy the producing kernel wrote (MFMA, fp32 accumulate)
+//   MN_SEQ_ARITH_BF16, 9 .. 64 rows  mn_skinny_gemm's weight-streaming MFMA route on bf16 hi/lo rows (fp32-class products)
+//   MN_SEQ_ARITH_BF16, M > 64        mn_gemm_bf16 on the bf16 copy the producing kernel wrote (MFMA, fp32 accumulate)
 //   MN_SEQ_ARITH_F32, or a K that is no multiple of 8 / an unaligned weight: mn_gemm_f32_batched (fp32 FMA tiles)
 // The per-head absorb (q W_uk) and expand (latent W_uv^T) products are batched over heads on the fp32 FMA kernel in both modes.
 #include <string.h>
@@ -18,14 +19,19 @@ inline size_t al(size_t n) { return (n + 255) & ~(size_t)255; }
 
 inline bool mfma_ok(const uint16_t* W, int K) { return K >= 8 && (K % 8) == 0 && (((uintptr_t)W) & 15) == 0; }
 
-// C fp32 [M, N] = A W^T + bias.  A16 (optional) = bf16 copy of A with row stride lda16.
+// C fp32 [M, N] = A W^T + bias.  A16 (optional) = bf16 copy of A with row stride lda16; gws / gws_bytes: scratch of the weight-streaming
+// MFMA route (mn_skinny_workspace_bytes).
 int linear(int arith, int M, const float* A, int64_t lda, const uint16_t* A16, int64_t lda16, const uint16_t* W, int N, int K,
-           const uint16_t* bias, float* C, int64_t ldc, void* stream) {
-  if (M <= 8 && mfma_ok(W, K)) {
+           const uint16_t* bias, float* C, int64_t ldc, void* gws, size_t gws_bytes, void* stream) {
+  // <= 8 rows: weight streaming on fp32 FMA.  9 .. 64 rows (bf16 arithmetic): the weight-streaming MFMA route on hi/lo rows — every
+  // weight byte once over all CUs, where the tiled GEMM would put a 32-row problem on N / 128 workgroups
+  const bool stream_mfma = arith == MN_SEQ_ARITH_BF16 && M > 8 && M <= 64 && gws && gws_bytes >= mn_skinny_workspace_bytes(M, N, K, MN_EPI_NONE);
+  if ((M <= 8 || stream_mfma) && mfma_ok(W, K)) {
     mn_skinny_args a;
     memset(&a, 0, sizeof(a));
     a.x = A; a.ldx = lda; a.w = W; a.ldw = K; a.bias = bias; a.out = C; a.ldo = ldc;
     a.M = M; a.N = N; a.K = K;
+    if (M > 8) { a.ws = gws; a.ws_bytes = gws_bytes; }
     return mn_skinny_gemm(&a, stream);
   }
   if (arith == MN_SEQ_ARITH_BF16 && A16 && mfma_ok(W, K) && (lda16 % 8) == 0 && (((uintptr_t)A16) & 15) == 0)
@@ -54,7 +60,7 @@ Dims layer_dims(const mn_seq_layer& l) {
 
 struct Plan {
   int n_in = 1, hd = 1, hv = 1, hr = 1, q_rank = 1, ff = 1;
-  size_t attn_ws = 0;
+  size_t attn_ws = 0, gemm_ws = 0;
 };
 
 Plan make_plan(const mn_seq_model* m, int M, int max_len) {
@@ -73,6 +79,15 @@ Plan make_plan(const mn_seq_model* m, int M, int max_len) {
     const int ks = mn_latent_attn_splits((int)mn_cdiv(M, RB), max_len, l.kv_rank);
     const size_t w = mn_latent_attn_workspace_bytes(M, l.heads, l.kv_rank, ks);
     if (w > p.attn_ws) p.attn_ws = w;
+    if (m->arith == MN_SEQ_ARITH_BF16 && M > 8 && M <= 64) {       // scratch of the weight-streaming MFMA route: the largest product of the stack
+      const int W = m->width;
+      const int shapes[6][2] = {{W, W}, {d.n_in, W}, {d.hd, d.q_rank}, {W, d.hv}, {W + d.ff, W}, {W, d.ff}};
+      for (const auto& nk : shapes) {
+        if (nk[0] < 1 || nk[1] < 8 || (nk[1] % 8) != 0) continue;
+        const size_t g = mn_skinny_workspace_bytes(M, nk[0], nk[1], MN_EPI_NONE);
+        if (g > p.gemm_ws) p.gemm_ws = g;
+      }
+    }
   }
   return p;
 }
@@ -96,7 +111,7 @@ extern "C" size_t mn_seq_workspace_bytes(const mn_seq_model* m, int M, int max_l
   n += al(R * W * 4);                       // sublayer result
   n += al(R * (W + p.ff) * 4);              // [gate pre-activation ; up] of the feed-forward
   n += al(R * p.ff * 4) + al(R * p.ff * 2); // activation + bf16
-  n += al(p.attn_ws);
+  n += al(p.attn_ws) + al(p.gemm_ws);
   return n;
 }
 
@@ -113,7 +128,7 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
   const Plan p = make_plan(m, M, max_len);
   const int W = m->width, arith = m->arith;
   const size_t R = (size_t)M;
-  const bool want16 = arith == MN_SEQ_ARITH_BF16 && M > 8;
+  const bool want16 = arith == MN_SEQ_ARITH_BF16 && M > 64;       // bf16 copies feed the tiled MFMA GEMM only
   char* wp = reinterpret_cast<char*>(workspace);
   auto take = [&](size_t bytes) { char* q = wp; wp += al(bytes); return q; };
   float* xr = (float*)take(R * W * 4);
@@ -135,6 +150,8 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
   float* af = (float*)take(R * p.ff * 4);
   uint16_t* afh = (uint16_t*)take(R * p.ff * 2);
   void* attn_ws = p.attn_ws ? take(p.attn_ws) : nullptr;
+  void* gws = p.gemm_ws ? take(p.gemm_ws) : nullptr;
+  const size_t gwb = p.gemm_ws;
   if (!want16) n1h = hh = cqh = atth = afh = nullptr;
   hipStream_t hs = mn_stream(stream);
   int rc;
@@ -151,14 +168,14 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
     float* tstate = st->taps ? st->taps + (size_t)li * taps_layer : nullptr;
     // ---- mixer sublayer ----
     MN_TRY(mn_affine_ln_rows(xr, W, l.norm1_w, l.norm1_b, m->eps, n1, W, n1h, W, M, W, stream));
-    MN_TRY(linear(arith, M, n1, W, n1h, W, l.rg1_w, W, W, l.rg1_b, g1, W, stream));
+    MN_TRY(linear(arith, M, n1, W, n1h, W, l.rg1_w, W, W, l.rg1_b, g1, W, gws, gwb, stream));
     MN_TRY(mn_tap_filter_rows(n1, W, l.taps_w, m->taps, tstate, row_seq, row_slot, row_back, hf, W, hh, W, M, W, stream));
     MN_TRY(mn_tap_state_update(n1, W, m->taps, tstate, row_seq, row_back, M, W, stream));
-    MN_TRY(linear(arith, M, hf, W, hh, W, l.w_in, d.n_in, W, nullptr, pin, d.n_in, stream));
+    MN_TRY(linear(arith, M, hf, W, hh, W, l.w_in, d.n_in, W, nullptr, pin, d.n_in, gws, gwb, stream));
     const float* qp; int64_t ldq; const float* gp = nullptr; int kv_off;
     if (l.kind == MN_SEQ_MIX_LATENT_Q) {
       MN_TRY(mn_rms_rows(pin, d.n_in, l.q_norm, m->eps, cq, l.q_rank, cqh, l.q_rank, nullptr, nullptr, 0, M, l.q_rank, stream));
-      MN_TRY(linear(arith, M, cq, l.q_rank, cqh, l.q_rank, l.w_uq, d.hd, l.q_rank, nullptr, qf, d.hd, stream));
+      MN_TRY(linear(arith, M, cq, l.q_rank, cqh, l.q_rank, l.w_uq, d.hd, l.q_rank, nullptr, qf, d.hd, gws, gwb, stream));
       qp = qf; ldq = d.hd; kv_off = l.q_rank;
     } else {
       qp = pin; ldq = d.n_in; gp = pin + d.hd; kv_off = d.hd + d.hv;
@@ -175,15 +192,15 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
     // expand: att[m, h, :] = W_uv[h] lat[m, h, :]  (* sigmoid(gate))
     MN_TRY(mn_gemm_f32_batched(lat, d.hr, l.kv_rank, l.w_uv, l.kv_rank, (int64_t)l.vdim * l.kv_rank, nullptr, att, d.hv, l.vdim, atth, d.hv,
                                l.vdim, gp, d.n_in, l.vdim, M, l.vdim, l.kv_rank, l.heads, 1.0f, stream));
-    MN_TRY(linear(arith, M, att, d.hv, atth, d.hv, l.w_o, W, d.hv, nullptr, yf, W, stream));
+    MN_TRY(linear(arith, M, att, d.hv, atth, d.hv, l.w_o, W, d.hv, nullptr, yf, W, gws, gwb, stream));
     MN_TRY(mn_gated_ln_residual(xr, W, g1, W, yf, W, l.norm1b_w, l.norm1b_b, m->eps, M, W, stream));
     // ---- feed-forward sublayer ----
     if (l.ff > 0) {
       const int nf = W + l.ff;
       MN_TRY(mn_affine_ln_rows(xr, W, l.norm2_w, l.norm2_b, m->eps, n1, W, n1h, W, M, W, stream));
-      MN_TRY(linear(arith, M, n1, W, n1h, W, l.w_ff_in, nf, W, l.b_ff_in, fin, nf, stream));
+      MN_TRY(linear(arith, M, n1, W, n1h, W, l.w_ff_in, nf, W, l.b_ff_in, fin, nf, gws, gwb, stream));
       MN_TRY(mn_polynorm_rows(fin + W, nf, l.act, m->eps, af, l.ff, afh, l.ff, M, l.ff, stream));
-      MN_TRY(linear(arith, M, af, l.ff, afh, l.ff, l.w_down, W, l.ff, nullptr, yf, W, stream));
+      MN_TRY(linear(arith, M, af, l.ff, afh, l.ff, l.w_down, W, l.ff, nullptr, yf, W, gws, gwb, stream));
       MN_TRY(mn_gated_ln_residual(xr, W, fin, nf, yf, W, l.norm2b_w, l.norm2b_b, m->eps, M, W, stream));
     }
     if (trace) {
@@ -206,7 +223,7 @@ extern "C" int mn_seq_logits(const float* hidden, int64_t ldh, int M, const uint
     if (rc != MN_OK) return rc;
     h16 = (const uint16_t*)workspace;
   }
-  int rc = linear(arith, M, hidden, ldh, h16, K, Wt, V, K, nullptr, out, ldo, stream);
+  int rc = linear(arith, M, hidden, ldh, h16, K, Wt, V, K, nullptr, out, ldo, nullptr, 0, stream);
   if (rc != MN_OK) return rc;
   if (cap > 0.f) rc = mn_softcap_rows(out, ldo, M, V, cap, stream);
   return rc;

@@ -298,11 +298,17 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 a) {
   }
 }
 
-// C[z][m, n] = alpha * A[z][m, :] . W[z][n, :] (+ bias) (* sigmoid(G)) for M <= 8 rows: one wave per output column, lanes over K
+// C[z][m, n] = alpha * A[z][m, :] . W[z][n, :] (+ bias) (* sigmoid(G)) for few rows: one wave per output column and MM rows, lanes over K
 template <int MM>
 __global__ __launch_bounds__(256) void gemv_f32_kernel(GemmF32 a) {
   const int z = blockIdx.z, n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (n >= a.N) return;
+  const int m0 = blockIdx.y * MM;                       // this workgroup's rows: m0 .. m0 + MM - 1
+  a.M -= m0;
+  a.A += (int64_t)m0 * a.lda;
+  if (a.C) a.C += (int64_t)m0 * a.ldc;
+  if (a.C16) a.C16 += (int64_t)m0 * a.ldc16;
+  if (a.G) a.G += (int64_t)m0 * a.ldg;
   const float* A = a.A + (int64_t)z * a.a_bs;
   const bf16_t* Wr = a.W + (int64_t)z * a.w_bs + (int64_t)n * a.ldw;
   float acc[MM];
@@ -688,10 +694,9 @@ extern "C" int mn_gemm_f32_batched(const float* A, int64_t lda, int64_t a_bs, co
   MN_CHECK_ARG(A && W && (C || C16) && M >= 1 && N >= 1 && K >= 1 && batch >= 1 && batch <= 65535, "mn_gemm_f32_batched: bad args");
   GemmF32 a{A, lda, a_bs, W, ldw, w_bs, bias, C, ldc, c_bs, C16, ldc16, c16_bs, G, ldg, g_bs, M, N, K, alpha};
   hipStream_t st = mn_stream(stream);
-  if (M <= 8) {
-    MN_CHECK_ARG(mn_cdiv(N, 4) <= 0x7fffffff, "mn_gemm_f32_batched: too many columns");
+  if (M <= 64) {                                         // decode-sized steps: the weights of a head are a few hundred KiB, rows in groups of 8
     if (M <= 2) hipLaunchKernelGGL((gemv_f32_kernel<2>), dim3((unsigned)mn_cdiv(N, 4), 1, (unsigned)batch), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((gemv_f32_kernel<8>), dim3((unsigned)mn_cdiv(N, 4), 1, (unsigned)batch), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemv_f32_kernel<8>), dim3((unsigned)mn_cdiv(N, 4), (unsigned)mn_cdiv(M, 8), (unsigned)batch), dim3(256), 0, st, a);
   } else if (M <= 16) {
     hipLaunchKernelGGL((gemm_f32_kernel<1>), dim3((unsigned)mn_cdiv(N, 64), 1, (unsigned)batch), dim3(256), 0, st, a);
   } else {

@@ -138,7 +138,7 @@ def test_tap_filter_with_state():
 def test_fp32_batched_product():
     from ming_univision_amd._lib import check, current_stream, lib, ptr
     g = torch.Generator().manual_seed(2)
-    for M, N, K, B in ((1, 40, 24, 3), (5, 7, 3, 1), (16, 64, 16, 2), (17, 65, 17, 2), (200, 130, 72, 5)):
+    for M, N, K, B in ((1, 40, 24, 3), (5, 7, 3, 1), (16, 64, 16, 2), (17, 65, 17, 2), (33, 70, 130, 3), (64, 9, 40, 1), (65, 66, 20, 2), (200, 130, 72, 5)):
         a = torch.randn(M, B * K, generator=g)
         w = _bf(torch.randn(B, N, K, generator=g))
         bias = _bf(torch.randn(N, generator=g))
@@ -329,14 +329,16 @@ def test_long_decoding():
 
 
 def test_bf16_arithmetic():
-    """Serving arithmetic: portions above 8 rows take the bf16 MFMA products (3e-2 of the logits' scale against the oracle), rows
-    fed one by one take fp32 FMA and stay at fp32 accuracy."""
-    cfg, sd, dec = make("ones", arith="bf16")
-    t = toks(cfg, 120)
-    ref = O.logits_of(cfg, sd, t)
-    assert err(run_portions(dec, 0, t, [120]), ref) < 3e-2
-    assert err(run_portions(dec, 0, t, [60, 30, 30]), ref) < 3e-2
-    assert err(run_portions(dec, 0, t[:40], [1] * 40), ref[:40]) < 1e-4
+    """Serving arithmetic: portions above 64 rows take the bf16 MFMA products (3e-2 of the logits' scale against the oracle),
+    portions of 9 .. 64 rows the weight-streaming MFMA route on hi/lo rows, rows fed a few at a time fp32 FMA."""
+    for name in ("ones", "mixed"):                      # "mixed": some products have a K that is no multiple of 8 and stay on fp32 FMA
+        cfg, sd, dec = make(name, arith="bf16")
+        t = toks(cfg, 150)
+        ref = O.logits_of(cfg, sd, t)
+        assert err(run_portions(dec, 0, t, [150]), ref) < 3e-2                   # tiled MFMA GEMM (above 64 rows)
+        assert err(run_portions(dec, 0, t, [70, 40, 31, 9]), ref) < 3e-2         # + the weight-streaming MFMA route (9 .. 64 rows)
+        assert err(run_portions(dec, 0, t[:40], [1] * 40), ref[:40]) < 1e-4      # fp32 FMA
+        assert err(run_portions(dec, 0, t[:64], [12, 20, 32]), ref[:64]) < 5e-3  # hi/lo rows (measured 2e-3; the tiled GEMM 6e-3 .. 9e-3)
 
 
 def test_greedy_generation_entry_point():
