@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MN_VERSION 125 /* 0.1.25: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
+#define MN_VERSION 126 /* 0.1.26: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
                           mn_llm and mn_llm_tp (zero = bf16: callers of 0.1.10 that zero-fill the structs are unchanged),
                           mn_quant_fp8_rows / mn_dequant_fp8_rows / mn_stream_mfma_w8 / mn_stream_mfma_grouped_w8 */
 
@@ -753,7 +753,7 @@ MN_API int mn_gemm256_f8(const uint8_t* A, int64_t lda, const float* a_scale, co
 MN_API int mn_gemm256_f8_slices(int K, int ksplit);
 
 /* ------------------------------------------------------------------------------------------
- * 9. Latent-cache sequence models (0.1.25): decoder stacks whose attention layers cache one low-rank latent per token instead of
+ * 9. Latent-cache sequence models (0.1.26): decoder stacks whose attention layers cache one low-rank latent per token instead of
  *    keys and values (keys and values of every head are linear maps of it, so queries are absorbed into latent space and the
  *    attention runs against the latents themselves), with a short causal per-channel filter in front of the mixer, sigmoid-gated
  *    sublayer results that are normalised before the residual add, and a polynomial-of-unit-norms feed-forward activation.
@@ -783,6 +783,13 @@ MN_API int mn_tap_filter_rows(const float* x, int64_t ldx, const uint16_t* w, in
                               int M, int n, void* stream);
 MN_API int mn_tap_state_update(const float* x, int64_t ldx, int taps, float* state, const int32_t* row_seq, const int32_t* row_back,
                                int M, int n, void* stream);
+/* Decode rows — every row ALONE in its sequence within the call — in one launch, up to three stages: (g given) x += LN(sigmoid(g) y;
+ * wa, ba); n_out = LN(x; wb, bb); (h given) h = n_out + the tap filter over the sequence's state, and the state moves on by this row
+ * (mn_tap_filter_rows + mn_tap_state_update for one-row sequences).  Rows of at most 8192 values. */
+MN_API int mn_gated_norm_filter_rows(float* x, int64_t ldx, const float* g, int64_t ldg, const float* y, int64_t ldy, const uint16_t* wa,
+                                     const uint16_t* ba, const uint16_t* wb, const uint16_t* bb, float eps, float* n_out, int64_t ldn,
+                                     const uint16_t* taps_w, int taps, float* state, const int32_t* row_seq, const int32_t* row_slot,
+                                     float* h, int64_t ldh, int M, int n, void* stream);
 MN_API int mn_softcap_rows(float* z, int64_t ld, int M, int n, float cap, void* stream);
 /* C[z] = alpha * A[z] W[z]^T (+ bias) (* sigmoid(G[z])) for z < batch, operands of batch entry z at base + z * (their _bs stride):
  * fp32 FMA, any M / N / K.  C (fp32) and C16 (bf16 copy) are both optional outputs. */
@@ -850,9 +857,10 @@ MN_API size_t mn_sizeof_seq_state(void);
  * attends); blk_tab / n_blk as in mn_latent_attn; max_len >= every row_len.  Appends the latents, advances the filter states.
  * out fp32 [M, width]: the final norm's output.  trace (optional) fp32 [n_layers, M, width]: the residual stream after every layer. */
 MN_API size_t mn_seq_workspace_bytes(const mn_seq_model* m, int M, int max_len);
+enum { MN_SEQ_ROWS_DISTINCT = 1 };   /* flags: every row is alone in its sequence (a decode step): gate / norm / filter launches are fused */
 MN_API int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
                        const int32_t* row_slot, const int32_t* row_back, const int32_t* row_len, const int32_t* blk_tab, int n_blk,
-                       int max_len, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
+                       int max_len, int flags, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
 /* logits fp32 [M, V] = hidden W^T by the step's product routing (arith as in mn_seq_model), then the soft cap (cap <= 0: none);
  * workspace: M * K * 2 bytes (the bf16 operand of the MFMA route) */
 MN_API int mn_seq_logits(const float* hidden, int64_t ldh, int M, const uint16_t* W, int V, int K, float cap, int arith, float* out,

@@ -283,7 +283,8 @@ SYMBOLS = {
     "mn_latent_attn": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _sz, _p]),
     "mn_latent_attn_ex": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _sz, _i, _p]),
     "mn_seq_workspace_bytes": (_sz, [C.POINTER(SeqModel), _i, _i]),
-    "mn_seq_step": (_i, [C.POINTER(SeqModel), C.POINTER(SeqState), _p, _i64, _i, _p, _p, _p, _p, _p, _i, _i, _p, _p, _p, _sz, _p]),
+    "mn_seq_step": (_i, [C.POINTER(SeqModel), C.POINTER(SeqState), _p, _i64, _i, _p, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
+    "mn_gated_norm_filter_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _f, _p, _i64, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "mn_seq_logits": (_i, [_p, _i64, _i, _p, _i, _i, _f, _i, _p, _i64, _p, _sz, _p]),
     "mn_semdec_step": (_i, [C.POINTER(SemDec), _p, _i, _p, _p, _p, _p, _i, _i64, _p, _p, _p, _sz, _p]),
 }
@@ -305,7 +306,7 @@ def lib():
         fn = getattr(handle, name)  # AttributeError if the symbol is missing
         fn.restype = res
         fn.argtypes = args
-    if handle.mn_version() < 125:
+    if handle.mn_version() < 126:
         raise RuntimeError("libmingnative.so is too old")
     check_struct_layouts(handle)
     _lib = handle

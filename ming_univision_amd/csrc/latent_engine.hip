@@ -117,7 +117,7 @@ extern "C" size_t mn_seq_workspace_bytes(const mn_seq_model* m, int M, int max_l
 
 extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
                            const int32_t* row_slot, const int32_t* row_back, const int32_t* row_len, const int32_t* blk_tab, int n_blk,
-                           int max_len, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream) {
+                           int max_len, int flags, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream) {
   MN_CHECK_ARG(m && st && m->layers && st->latent && x && row_seq && row_slot && row_back && row_len && blk_tab && out && workspace,
                "mn_seq_step: null pointer");
   MN_CHECK_ARG(M >= 1 && M <= 65535 && n_blk >= 1 && n_blk <= M && m->width >= 1 && m->n_layers >= 1 && m->taps >= 1,
@@ -159,6 +159,28 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
   hipLaunchKernelGGL(copy_rows_kernel, dim3((unsigned)mn_cdiv(W, 256), (unsigned)M), dim3(256), 0, hs, x, ldx, xr, W);
   MN_CHECK_LAUNCH("mn_seq_step(copy)");
   const size_t taps_layer = (size_t)st->n_seq * (m->taps - 1) * W;
+  // A sublayer ends with x += LN(sigmoid(g) y) and the next one starts with LN(x) (+ the tap filter in front of a mixer).  On decode
+  // steps (MN_SEQ_ROWS_DISTINCT, no bf16 copies wanted) the end of one and the start of the next are ONE launch; otherwise the
+  // operators run one by one.  `pend` is a sublayer end that has not been applied to x yet.
+  const bool fuse = (flags & MN_SEQ_ROWS_DISTINCT) && !want16 && W <= 8192 && !trace;
+  struct Pending { const float* g = nullptr; int64_t ldg = 0; const uint16_t *w = nullptr, *b = nullptr; } pend;
+  // n_out = LN(x; wb, bb) after applying `pend`; with tstate / h_out also h = n + filter(n) and the state update
+  auto norm_stage = [&](const uint16_t* wb, const uint16_t* bb, float* n_out, uint16_t* n16, const uint16_t* taps_w, float* tstate,
+                        float* h_out, uint16_t* h16) -> int {
+    if (fuse) {
+      const int rc2 = mn_gated_norm_filter_rows(xr, W, pend.g, pend.ldg, yf, W, pend.w, pend.b, wb, bb, m->eps, n_out, W, taps_w, m->taps, tstate,
+                                                row_seq, row_slot, h_out, W, M, W, stream);
+      pend = Pending();
+      return rc2;
+    }
+    int rc2 = MN_OK;
+    if (pend.g) rc2 = mn_gated_ln_residual(xr, W, pend.g, pend.ldg, yf, W, pend.w, pend.b, m->eps, M, W, stream);
+    pend = Pending();
+    if (rc2 == MN_OK) rc2 = mn_affine_ln_rows(xr, W, wb, bb, m->eps, n_out, W, n16, W, M, W, stream);
+    if (rc2 == MN_OK && h_out) rc2 = mn_tap_filter_rows(n_out, W, taps_w, m->taps, tstate, row_seq, row_slot, row_back, h_out, W, h16, W, M, W, stream);
+    if (rc2 == MN_OK && h_out) rc2 = mn_tap_state_update(n_out, W, m->taps, tstate, row_seq, row_back, M, W, stream);
+    return rc2;
+  };
   for (int li = 0; li < m->n_layers; ++li) {
     const mn_seq_layer& l = m->layers[li];
     const Dims d = layer_dims(l);
@@ -167,10 +189,8 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
     float* arena = st->latent[l.arena];
     float* tstate = st->taps ? st->taps + (size_t)li * taps_layer : nullptr;
     // ---- mixer sublayer ----
-    MN_TRY(mn_affine_ln_rows(xr, W, l.norm1_w, l.norm1_b, m->eps, n1, W, n1h, W, M, W, stream));
+    MN_TRY(norm_stage(l.norm1_w, l.norm1_b, n1, n1h, l.taps_w, tstate, hf, hh));
     MN_TRY(linear(arith, M, n1, W, n1h, W, l.rg1_w, W, W, l.rg1_b, g1, W, gws, gwb, stream));
-    MN_TRY(mn_tap_filter_rows(n1, W, l.taps_w, m->taps, tstate, row_seq, row_slot, row_back, hf, W, hh, W, M, W, stream));
-    MN_TRY(mn_tap_state_update(n1, W, m->taps, tstate, row_seq, row_back, M, W, stream));
     MN_TRY(linear(arith, M, hf, W, hh, W, l.w_in, d.n_in, W, nullptr, pin, d.n_in, gws, gwb, stream));
     const float* qp; int64_t ldq; const float* gp = nullptr; int kv_off;
     if (l.kind == MN_SEQ_MIX_LATENT_Q) {
@@ -193,22 +213,24 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
     MN_TRY(mn_gemm_f32_batched(lat, d.hr, l.kv_rank, l.w_uv, l.kv_rank, (int64_t)l.vdim * l.kv_rank, nullptr, att, d.hv, l.vdim, atth, d.hv,
                                l.vdim, gp, d.n_in, l.vdim, M, l.vdim, l.kv_rank, l.heads, 1.0f, stream));
     MN_TRY(linear(arith, M, att, d.hv, atth, d.hv, l.w_o, W, d.hv, nullptr, yf, W, gws, gwb, stream));
-    MN_TRY(mn_gated_ln_residual(xr, W, g1, W, yf, W, l.norm1b_w, l.norm1b_b, m->eps, M, W, stream));
+    pend.g = g1; pend.ldg = W; pend.w = l.norm1b_w; pend.b = l.norm1b_b;
     // ---- feed-forward sublayer ----
     if (l.ff > 0) {
       const int nf = W + l.ff;
-      MN_TRY(mn_affine_ln_rows(xr, W, l.norm2_w, l.norm2_b, m->eps, n1, W, n1h, W, M, W, stream));
+      MN_TRY(norm_stage(l.norm2_w, l.norm2_b, n1, n1h, nullptr, nullptr, nullptr, nullptr));
       MN_TRY(linear(arith, M, n1, W, n1h, W, l.w_ff_in, nf, W, l.b_ff_in, fin, nf, gws, gwb, stream));
       MN_TRY(mn_polynorm_rows(fin + W, nf, l.act, m->eps, af, l.ff, afh, l.ff, M, l.ff, stream));
       MN_TRY(linear(arith, M, af, l.ff, afh, l.ff, l.w_down, W, l.ff, nullptr, yf, W, gws, gwb, stream));
-      MN_TRY(mn_gated_ln_residual(xr, W, fin, nf, yf, W, l.norm2b_w, l.norm2b_b, m->eps, M, W, stream));
+      pend.g = fin; pend.ldg = nf; pend.w = l.norm2b_w; pend.b = l.norm2b_b;
     }
-    if (trace) {
+    if (trace) {                                       // the trace wants x after the whole layer: apply the layer's last sublayer end now
+      MN_TRY(mn_gated_ln_residual(xr, W, pend.g, pend.ldg, yf, W, pend.w, pend.b, m->eps, M, W, stream));
+      pend = Pending();
       const hipError_t e = hipMemcpyAsync(trace + (size_t)li * R * W, xr, R * W * 4, hipMemcpyDeviceToDevice, hs);
       if (e != hipSuccess) { mn_set_error("mn_seq_step: trace copy: %s", hipGetErrorString(e)); return MN_ELAUNCH; }
     }
   }
-  MN_TRY(mn_affine_ln_rows(xr, W, m->final_w, m->final_b, m->eps, out, W, nullptr, 0, M, W, stream));
+  MN_TRY(norm_stage(m->final_w, m->final_b, out, nullptr, nullptr, nullptr, nullptr, nullptr));
 #undef MN_TRY
   return MN_OK;
 }

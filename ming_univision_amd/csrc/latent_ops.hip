@@ -298,6 +298,85 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 a) {
   }
 }
 
+// Decode rows (every row alone in its sequence), one workgroup per row, the row in registers, up to three stages in one launch:
+//   1 (g given)  x += LN(sigmoid(g) * y; wa, ba)          the previous sublayer's gate, norm and residual add
+//   2            n  = LN(x; wb, bb)                        this sublayer's input norm
+//   3 (h given)  h  = n + taps filter over the sequence's last inputs (from its state), and the state moves on by this row
+struct FusedRowArgs {
+  float* x; int64_t ldx;
+  const float* g; int64_t ldg;
+  const float* y; int64_t ldy;
+  const bf16_t *wa, *ba, *wb, *bb;
+  float eps;
+  float* n_out; int64_t ldn;
+  const bf16_t* taps_w; int taps;
+  float* state; const int32_t* row_seq; const int32_t* row_slot;
+  float* h; int64_t ldh;
+  int n;
+};
+
+template <int VPT>
+__global__ __launch_bounds__(256) void row_fused_kernel(FusedRowArgs a) {
+  __shared__ float red[8];
+  const int row = blockIdx.x, tid = threadIdx.x, n = a.n;
+  float xv[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = tid + 256 * i;
+    const float t = a.x[(int64_t)row * a.ldx + (c < n ? c : 0)];
+    xv[i] = c < n ? t : 0.f;
+  }
+  if (a.g) {
+    float t[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = tid + 256 * i, cc = c < n ? c : 0;
+      const float gv = a.g[(int64_t)row * a.ldg + cc], yv = a.y[(int64_t)row * a.ldy + cc];
+      t[i] = c < n ? sigmoid_f(gv) * yv : 0.f;
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) s += t[i];
+    const float mean = block_sum(s, red) / (float)n;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) { const float d = (tid + 256 * i < n) ? t[i] - mean : 0.f; q += d * d; }
+    const float rstd = 1.0f / sqrtf(block_sum(q, red) / (float)n + a.eps);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = tid + 256 * i;
+      if (c >= n) continue;
+      xv[i] += (t[i] - mean) * rstd * bf16_to_f32(a.wa[c]) + bf16_to_f32(a.ba[c]);
+      a.x[(int64_t)row * a.ldx + c] = xv[i];
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) s += xv[i];
+  const float mean = block_sum(s, red) / (float)n;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) { const float d = (tid + 256 * i < n) ? xv[i] - mean : 0.f; q += d * d; }
+  const float rstd = 1.0f / sqrtf(block_sum(q, red) / (float)n + a.eps);
+  const int seq = a.h ? a.row_seq[row] : 0, slot = a.h ? a.row_slot[row] : 0;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = tid + 256 * i;
+    if (c >= n) continue;
+    const float nv = (xv[i] - mean) * rstd * bf16_to_f32(a.wb[c]) + bf16_to_f32(a.bb[c]);
+    a.n_out[(int64_t)row * a.ldn + c] = nv;
+    if (a.h) {
+      float acc = nv + bf16_to_f32(a.taps_w[(int64_t)c * a.taps + (a.taps - 1)]) * nv;
+      float* st = a.state + (int64_t)seq * (a.taps - 1) * n + c;
+      for (int k = 1; k < a.taps; ++k)
+        if (slot - k >= 0) acc += bf16_to_f32(a.taps_w[(int64_t)c * a.taps + (a.taps - 1 - k)]) * st[(int64_t)(k - 1) * n];
+      a.h[(int64_t)row * a.ldh + c] = acc;
+      for (int k = a.taps - 2; k >= 1; --k) st[(int64_t)k * n] = st[(int64_t)(k - 1) * n];
+      if (a.taps > 1) st[0] = nv;
+    }
+  }
+}
+
 // C[z][m, n] = alpha * A[z][m, :] . W[z][n, :] (+ bias) (* sigmoid(G)) for few rows: one wave per output column and MM rows, lanes over K
 template <int MM>
 __global__ __launch_bounds__(256) void gemv_f32_kernel(GemmF32 a) {
@@ -678,6 +757,23 @@ extern "C" int mn_tap_state_update(const float* x, int64_t ldx, int taps, float*
   hipLaunchKernelGGL(tap_state_kernel, dim3((unsigned)mn_cdiv(n, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), x, ldx, taps, state,
                      row_seq, row_back, M, n);
   MN_CHECK_LAUNCH("mn_tap_state_update");
+  return MN_OK;
+}
+
+extern "C" int mn_gated_norm_filter_rows(float* x, int64_t ldx, const float* g, int64_t ldg, const float* y, int64_t ldy, const uint16_t* wa,
+                                         const uint16_t* ba, const uint16_t* wb, const uint16_t* bb, float eps, float* n_out, int64_t ldn,
+                                         const uint16_t* taps_w, int taps, float* state, const int32_t* row_seq, const int32_t* row_slot,
+                                         float* h, int64_t ldh, int M, int n, void* stream) {
+  MN_CHECK_ARG(x && wb && bb && n_out && M >= 1 && n >= 1 && n <= 8192, "mn_gated_norm_filter_rows: bad args (rows of at most 8192 values)");
+  MN_CHECK_ARG(!g || (y && wa && ba), "mn_gated_norm_filter_rows: the gated stage needs y and its norm");
+  MN_CHECK_ARG(!h || (taps_w && taps >= 1 && (state || taps == 1) && row_seq && row_slot), "mn_gated_norm_filter_rows: the filter stage needs its state");
+  const FusedRowArgs a{x, ldx, g, ldg, y, ldy, wa, ba, wb, bb, eps, n_out, ldn, taps_w, taps, state, row_seq, row_slot, h, ldh, n};
+  const int vpt = (n + 255) / 256;
+  hipStream_t st = mn_stream(stream);
+#define MN_RF(V_) hipLaunchKernelGGL((row_fused_kernel<V_>), dim3((unsigned)M), dim3(256), 0, st, a)
+  if (vpt <= 1) MN_RF(1); else if (vpt <= 2) MN_RF(2); else if (vpt <= 4) MN_RF(4); else if (vpt <= 8) MN_RF(8); else if (vpt <= 16) MN_RF(16); else MN_RF(32);
+#undef MN_RF
+  MN_CHECK_LAUNCH("mn_gated_norm_filter_rows");
   return MN_OK;
 }
 

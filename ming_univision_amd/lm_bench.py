@@ -73,7 +73,7 @@ def run_pizitar(s, T, batches, n_dec):
             slot = torch.full((B,), T, dtype=torch.int32, device=dev)
             ln = slot + 1
             for i in range(n_dec):
-                dec.step(xb, row_seq, slot, back, ln, blk, T + i + 1)
+                dec.step(xb, row_seq, slot, back, ln, blk, T + i + 1, distinct=True)
                 check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
         out[f"decode_b{B}_tokens_per_s"] = B * n_dec / _time(loop, 2, 1)
         slot_g = torch.full((B,), T, dtype=torch.int32, device=dev)

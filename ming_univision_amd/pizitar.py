@@ -184,12 +184,13 @@ class PizitarDecoder:
             self._ws[key] = torch.empty(need, dtype=torch.uint8, device=self.device)
         return self._ws[key]
 
-    def step(self, x, row_seq, row_slot, row_back, row_len, blk_tab, max_len, out=None, trace=None, ws=None):
+    def step(self, x, row_seq, row_slot, row_back, row_len, blk_tab, max_len, out=None, trace=None, ws=None, distinct=False):
         """One pass of the stack over M rows.  x fp32 [M, width] (input embeddings); int32 device arrays per row (row r is
         position row_slot[r] of cache sequence row_seq[r], preceded in this pass by row_back[r] rows of its sequence, and attends
         row_len[r] = row_slot[r] + 1 slots); blk_tab int32 [n_blk, 2] cuts the rows into runs of <= block_rows consecutive rows of
         one sequence; max_len (host int) >= every row_len.  Appends the rows' latents and advances the filter states.
         trace: optional fp32 [layers, M, width] that receives the residual stream after every layer.
+        distinct: every row is alone in its sequence (a decode step): the step fuses its gate / norm / filter launches.
         Returns the final norm's output [M, width] fp32."""
         M = x.shape[0]
         assert x.dtype == torch.float32 and x.is_cuda and x.stride(1) == 1 and x.shape[1] == self.cfg.width and 1 <= M <= MAX_ROWS
@@ -204,7 +205,7 @@ class PizitarDecoder:
         if ws is None:
             ws = self._workspace(M, max_len)
         check(lib().mn_seq_step(C.byref(self.struct), C.byref(self.state), ptr(x), x.stride(0), M, ptr(row_seq), ptr(row_slot),
-                                ptr(row_back), ptr(row_len), ptr(blk_tab), blk_tab.shape[0], int(max_len), ptr(out), ptr(trace),
+                                ptr(row_back), ptr(row_len), ptr(blk_tab), blk_tab.shape[0], int(max_len), 1 if distinct else 0, ptr(out), ptr(trace),
                                 ptr(ws), ws.numel(), current_stream()), "mn_seq_step")
         return out
 
@@ -227,7 +228,7 @@ class PizitarDecoder:
             if trace:
                 ptr_tr = torch.empty(len(self.cfg.layers), r1 - r0, self.cfg.width, dtype=torch.float32, device=self.device)
             self.step(x[r0:r1], dev["row_seq"], dev["row_slot"], dev["row_back"], dev["row_len"], dev["blk_tab"], tabs["max_len"],
-                      out=out[r0:r1], trace=ptr_tr)
+                      out=out[r0:r1], trace=ptr_tr, distinct=all(n == 1 for _, n, _ in part))
             if trace:
                 tr[:, r0:r1] = ptr_tr
         return (out, tr) if trace else out
@@ -295,7 +296,7 @@ class DecodeGraph:
         self.bound, self.graph = 0, None
 
     def _body(self):
-        self.dec.step(self.x, self.row_seq, self.slot, self.back, self.len, self.blk, self.bound, out=self.out, ws=self.ws)
+        self.dec.step(self.x, self.row_seq, self.slot, self.back, self.len, self.blk, self.bound, out=self.out, ws=self.ws, distinct=True)
         check(lib().mn_rows_advance(ptr(self.slot), ptr(self.len), None, self.B, 1, current_stream()), "mn_rows_advance")
 
     def run(self, x, max_len):
@@ -367,7 +368,7 @@ class PizitarForCausalLM:
                 if graph is not None:
                     hidden = graph.run(dec.embed(tok), max(lens) + i + 1)
                 else:
-                    hidden = dec.step(dec.embed(tok), row_seq, slot, back, ln, blk, max(lens) + i + 1)
+                    hidden = dec.step(dec.embed(tok), row_seq, slot, back, ln, blk, max(lens) + i + 1, distinct=True)
                     check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
             out = torch.stack(toks, 1).tolist()
         finally:

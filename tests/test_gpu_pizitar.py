@@ -135,6 +135,41 @@ def test_tap_filter_with_state():
                 at[s] += c
 
 
+def test_fused_decode_rows():
+    """The one-launch form of a sublayer boundary for rows that are alone in their sequences (gate / norm / residual of the last
+    sublayer, the next input norm, the tap filter with its state) against the oracle's functions, fed row by row."""
+    from ming_univision_amd._lib import check, current_stream, lib, ptr
+    g = torch.Generator().manual_seed(3)
+    for n, taps, eps in ((44, 1, 1e-5), (192, 4, 1e-6), (1000, 3, 1e-5), (4100, 2, 1e-6)):
+        wa, ba, wb, bb = (_bf(1 + 0.3 * torch.randn(n, generator=g)) for _ in range(4))
+        tw = _bf(torch.randn(n, taps, generator=g))
+        steps, seqs = 6, [2, 0]                                      # two sequences, one row each per call
+        x0 = torch.randn(len(seqs), n, generator=g)
+        gs, ys = torch.randn(steps, len(seqs), n, generator=g), torch.randn(steps, len(seqs), n, generator=g)
+        dev = [t.cuda() for t in (wa, ba, wb, bb, tw)]
+        state = torch.full((3, max(taps - 1, 1), n), 5.0, device="cuda")
+        row_seq = torch.tensor(seqs, dtype=torch.int32, device="cuda")
+        x = x0.cuda()
+        xr, hist = x0.double().clone(), [[] for _ in seqs]
+        for t in range(steps):
+            slot = torch.full((len(seqs),), t, dtype=torch.int32, device="cuda")
+            gd, yd = gs[t].cuda(), ys[t].cuda()
+            nout, h = torch.empty_like(x), torch.empty_like(x)
+            gated = t % 2 == 1                                       # with and without the first stage
+            check(lib().mn_gated_norm_filter_rows(ptr(x), n, ptr(gd) if gated else None, n, ptr(yd), n, ptr(dev[0]), ptr(dev[1]), ptr(dev[2]),
+                                                  ptr(dev[3]), eps, ptr(nout), n, ptr(dev[4]), taps, ptr(state), ptr(row_seq), ptr(slot),
+                                                  ptr(h), n, len(seqs), n, current_stream()))
+            if gated:
+                xr = xr + O.affine_layer_norm(torch.sigmoid(gs[t].double()) * ys[t].double(), wa.double(), ba.double(), eps)
+            nr = O.affine_layer_norm(xr, wb.double(), bb.double(), eps)
+            assert err(x, xr) < 1e-5 and err(nout, nr) < 1e-5, (n, t)
+            for k in range(len(seqs)):
+                hist[k].append(nr[k])
+                seqn = torch.stack(hist[k])
+                want = (seqn + O.causal_tap_filter(seqn, tw.double()))[-1]
+                assert err(h[k], want) < 1e-5, (n, taps, t, k)
+
+
 def test_fp32_batched_product():
     from ming_univision_amd._lib import check, current_stream, lib, ptr
     g = torch.Generator().manual_seed(2)
