@@ -785,7 +785,7 @@ MN_API int mn_tap_state_update(const float* x, int64_t ldx, int taps, float* sta
                                int M, int n, void* stream);
 /* Decode rows — every row ALONE in its sequence within the call — in one launch, up to three stages: (g given) x += LN(sigmoid(g) y;
  * wa, ba); n_out = LN(x; wb, bb); (h given) h = n_out + the tap filter over the sequence's state, and the state moves on by this row
- * (mn_tap_filter_rows + mn_tap_state_update for one-row sequences).  Rows of at most 8192 values. */
+ * (mn_tap_filter_rows + mn_tap_state_update for one-row sequences).  Rows of at most 4096 values, at most 8 taps. */
 MN_API int mn_gated_norm_filter_rows(float* x, int64_t ldx, const float* g, int64_t ldg, const float* y, int64_t ldy, const uint16_t* wa,
                                      const uint16_t* ba, const uint16_t* wb, const uint16_t* bb, float eps, float* n_out, int64_t ldn,
                                      const uint16_t* taps_w, int taps, float* state, const int32_t* row_seq, const int32_t* row_slot,

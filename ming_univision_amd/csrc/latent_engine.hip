@@ -162,7 +162,7 @@ extern "C" int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const 
   // A sublayer ends with x += LN(sigmoid(g) y) and the next one starts with LN(x) (+ the tap filter in front of a mixer).  On decode
   // steps (MN_SEQ_ROWS_DISTINCT, no bf16 copies wanted) the end of one and the start of the next are ONE launch; otherwise the
   // operators run one by one.  `pend` is a sublayer end that has not been applied to x yet.
-  const bool fuse = (flags & MN_SEQ_ROWS_DISTINCT) && !want16 && W <= 8192 && !trace;
+  const bool fuse = (flags & MN_SEQ_ROWS_DISTINCT) && !want16 && W <= 4096 && m->taps <= 8 && !trace;
   struct Pending { const float* g = nullptr; int64_t ldg = 0; const uint16_t *w = nullptr, *b = nullptr; } pend;
   // n_out = LN(x; wb, bb) after applying `pend`; with tstate / h_out also h = n + filter(n) and the state update
   auto norm_stage = [&](const uint16_t* wb, const uint16_t* bb, float* n_out, uint16_t* n16, const uint16_t* taps_w, float* tstate,

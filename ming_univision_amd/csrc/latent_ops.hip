@@ -315,16 +315,27 @@ struct FusedRowArgs {
   int n;
 };
 
-template <int VPT>
+constexpr int FUSED_MAX_TAPS = 8;
+
+template <int VPT, bool FILTER>
 __global__ __launch_bounds__(256) void row_fused_kernel(FusedRowArgs a) {
   __shared__ float red[8];
   const int row = blockIdx.x, tid = threadIdx.x, n = a.n;
   float xv[VPT];
+  // everything the row needs from memory is requested before the first store: the state is float like the outputs, so a load
+  // placed after a store would wait its turn, one round trip per value
+  float sv[FILTER ? VPT : 1][FUSED_MAX_TAPS - 1];
+  const int seq = FILTER ? a.row_seq[row] : 0, slot = FILTER ? a.row_slot[row] : 0;
+  float* const st0 = FILTER ? a.state + (int64_t)seq * (a.taps - 1) * n : nullptr;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    const int c = tid + 256 * i;
-    const float t = a.x[(int64_t)row * a.ldx + (c < n ? c : 0)];
+    const int c = tid + 256 * i, cc = c < n ? c : 0;
+    const float t = a.x[(int64_t)row * a.ldx + cc];
     xv[i] = c < n ? t : 0.f;
+    if (FILTER) {
+#pragma unroll
+      for (int k = 1; k < FUSED_MAX_TAPS; ++k) sv[i][k - 1] = (k < a.taps) ? st0[(int64_t)(k - 1) * n + cc] : 0.f;
+    }
   }
   if (a.g) {
     float t[VPT];
@@ -358,20 +369,23 @@ __global__ __launch_bounds__(256) void row_fused_kernel(FusedRowArgs a) {
 #pragma unroll
   for (int i = 0; i < VPT; ++i) { const float d = (tid + 256 * i < n) ? xv[i] - mean : 0.f; q += d * d; }
   const float rstd = 1.0f / sqrtf(block_sum(q, red) / (float)n + a.eps);
-  const int seq = a.h ? a.row_seq[row] : 0, slot = a.h ? a.row_slot[row] : 0;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int c = tid + 256 * i;
     if (c >= n) continue;
     const float nv = (xv[i] - mean) * rstd * bf16_to_f32(a.wb[c]) + bf16_to_f32(a.bb[c]);
     a.n_out[(int64_t)row * a.ldn + c] = nv;
-    if (a.h) {
-      float acc = nv + bf16_to_f32(a.taps_w[(int64_t)c * a.taps + (a.taps - 1)]) * nv;
-      float* st = a.state + (int64_t)seq * (a.taps - 1) * n + c;
-      for (int k = 1; k < a.taps; ++k)
-        if (slot - k >= 0) acc += bf16_to_f32(a.taps_w[(int64_t)c * a.taps + (a.taps - 1 - k)]) * st[(int64_t)(k - 1) * n];
+    if (FILTER) {
+      const bf16_t* tw = a.taps_w + (int64_t)c * a.taps;
+      float acc = nv + bf16_to_f32(tw[a.taps - 1]) * nv;
+#pragma unroll
+      for (int k = 1; k < FUSED_MAX_TAPS; ++k)
+        if (k < a.taps && slot - k >= 0) acc += bf16_to_f32(tw[a.taps - 1 - k]) * sv[i][k - 1];
       a.h[(int64_t)row * a.ldh + c] = acc;
-      for (int k = a.taps - 2; k >= 1; --k) st[(int64_t)k * n] = st[(int64_t)(k - 1) * n];
+      float* st = st0 + c;
+#pragma unroll
+      for (int k = FUSED_MAX_TAPS - 2; k >= 1; --k)
+        if (k < a.taps - 1) st[(int64_t)k * n] = sv[i][k - 1];
       if (a.taps > 1) st[0] = nv;
     }
   }
@@ -764,14 +778,19 @@ extern "C" int mn_gated_norm_filter_rows(float* x, int64_t ldx, const float* g, 
                                          const uint16_t* ba, const uint16_t* wb, const uint16_t* bb, float eps, float* n_out, int64_t ldn,
                                          const uint16_t* taps_w, int taps, float* state, const int32_t* row_seq, const int32_t* row_slot,
                                          float* h, int64_t ldh, int M, int n, void* stream) {
-  MN_CHECK_ARG(x && wb && bb && n_out && M >= 1 && n >= 1 && n <= 8192, "mn_gated_norm_filter_rows: bad args (rows of at most 8192 values)");
+  MN_CHECK_ARG(x && wb && bb && n_out && M >= 1 && n >= 1 && n <= 4096, "mn_gated_norm_filter_rows: bad args (rows of at most 4096 values)");
   MN_CHECK_ARG(!g || (y && wa && ba), "mn_gated_norm_filter_rows: the gated stage needs y and its norm");
-  MN_CHECK_ARG(!h || (taps_w && taps >= 1 && (state || taps == 1) && row_seq && row_slot), "mn_gated_norm_filter_rows: the filter stage needs its state");
+  MN_CHECK_ARG(!h || (taps_w && taps >= 1 && taps <= FUSED_MAX_TAPS && (state || taps == 1) && row_seq && row_slot),
+               "mn_gated_norm_filter_rows: the filter stage needs its state and at most %d taps", FUSED_MAX_TAPS);
   const FusedRowArgs a{x, ldx, g, ldg, y, ldy, wa, ba, wb, bb, eps, n_out, ldn, taps_w, taps, state, row_seq, row_slot, h, ldh, n};
   const int vpt = (n + 255) / 256;
   hipStream_t st = mn_stream(stream);
-#define MN_RF(V_) hipLaunchKernelGGL((row_fused_kernel<V_>), dim3((unsigned)M), dim3(256), 0, st, a)
-  if (vpt <= 1) MN_RF(1); else if (vpt <= 2) MN_RF(2); else if (vpt <= 4) MN_RF(4); else if (vpt <= 8) MN_RF(8); else if (vpt <= 16) MN_RF(16); else MN_RF(32);
+#define MN_RF(V_)                                                                                                    \
+  do {                                                                                                               \
+    if (h) hipLaunchKernelGGL((row_fused_kernel<V_, true>), dim3((unsigned)M), dim3(256), 0, st, a);                 \
+    else hipLaunchKernelGGL((row_fused_kernel<V_, false>), dim3((unsigned)M), dim3(256), 0, st, a);                  \
+  } while (0)
+  if (vpt <= 1) MN_RF(1); else if (vpt <= 2) MN_RF(2); else if (vpt <= 4) MN_RF(4); else if (vpt <= 8) MN_RF(8); else MN_RF(16);
 #undef MN_RF
   MN_CHECK_LAUNCH("mn_gated_norm_filter_rows");
   return MN_OK;
