@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MN_VERSION 126 /* 0.1.26: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
+#define MN_VERSION 127 /* 0.1.27: parallel-mixer sequence models (section 10).  0.1.26: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
                           mn_llm and mn_llm_tp (zero = bf16: callers of 0.1.10 that zero-fill the structs are unchanged),
                           mn_quant_fp8_rows / mn_dequant_fp8_rows / mn_stream_mfma_w8 / mn_stream_mfma_grouped_w8 */
 
@@ -58,7 +58,8 @@ MN_API int mn_num_cus(void);
  * mn_struct_layout(which, offsets, cap) writes offsetof(every field, in declaration order) into offsets[0 .. min(n, cap)) and
  * returns the field count n (MN_EINVAL for an unknown `which`). */
 enum mn_struct_id { MN_STRUCT_SKINNY_ARGS = 0, MN_STRUCT_RF_HEAD = 1, MN_STRUCT_LLM = 2, MN_STRUCT_SEMDEC = 3, MN_STRUCT_TP_COMM = 4,
-                    MN_STRUCT_LLM_TP = 5, MN_STRUCT_SEQ_LAYER = 6, MN_STRUCT_SEQ_MODEL = 7, MN_STRUCT_SEQ_STATE = 8 };
+                    MN_STRUCT_LLM_TP = 5, MN_STRUCT_SEQ_LAYER = 6, MN_STRUCT_SEQ_MODEL = 7, MN_STRUCT_SEQ_STATE = 8,
+                    MN_STRUCT_PMIX_LAYER = 9, MN_STRUCT_PMIX_MODEL = 10, MN_STRUCT_PMIX_STATE = 11 };
 MN_API size_t mn_sizeof_skinny_args(void);
 MN_API size_t mn_sizeof_rf_head(void);
 MN_API size_t mn_sizeof_llm(void);
@@ -865,6 +866,120 @@ MN_API int mn_seq_step(const mn_seq_model* m, const mn_seq_state* st, const floa
  * workspace: M * K * 2 bytes (the bf16 operand of the MFMA route) */
 MN_API int mn_seq_logits(const float* hidden, int64_t ldh, int M, const uint16_t* W, int V, int K, float cap, int arith, float* out,
                          int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 10. Parallel-mixer sequence models (0.1.27): decoder stacks whose mixer is a windowed softmax attention (grouped key/value heads,
+ *     short causal filters on the projected q / k / v channels, rotary positions with optional YaRN frequencies on the first
+ *     `rot_dims` values of a head, unit-RMS queries and keys, a sliding window plus one mean key / value per whole block of `pool`
+ *     tokens before it) running beside a minGRU recurrence on the same input, both summed with fixed scales; RMS pre-norms with a
+ *     causal per-channel filter added to what each sublayer reads; a mixture-of-experts feed-forward (top-k softmax over the chosen
+ *     logits, optional sigmoid-gated shared expert); `x += mult * sublayer`.  A contiguous range of layers may run several times with
+ *     the same weights (each run owns its caches and states; the embedding rows are added again before every repeated pass).
+ *     Rows are fp32, weights bf16 [out, in]; every size and constant is a field or an argument.  The residual stream, norms,
+ *     angles, scores, softmax, router, recurrent state and cached keys / values are fp32 in both arithmetic modes (`arith` as in
+ *     section 9 chooses the matrix products).
+ * ------------------------------------------------------------------------------------------ */
+/* y_t = sum_j w[:, j] x_(t - taps + 1 + j): mn_tap_filter_rows without the added input (state and row arrays as there) */
+MN_API int mn_tap_conv_rows(const float* x, int64_t ldx, const uint16_t* w, int taps, const float* state, const int32_t* row_seq,
+                            const int32_t* row_slot, const int32_t* row_back, float* y, int64_t ldy, int M, int n, void* stream);
+/* x += mult * y (y may be NULL), then n_out = x / sqrt(mean(x^2) + eps) * w (n_out NULL: the add only); n16: optional bf16 copy */
+MN_API int mn_axpy_rms_rows(float* x, int64_t ldx, const float* y, int64_t ldy, float mult, const uint16_t* w, float eps, float* n_out,
+                            int64_t ldn, uint16_t* n16, int64_t ldn16, int M, int n, void* stream);
+/* Decode rows (every row alone in its sequence) in one launch: x += mult * y; n = RMS(x) w; h = n + the tap filter over the
+ * sequence's state (taps_w NULL: h = n), and the state moves on by this row.  Rows of at most 8192 values, at most 8 taps. */
+MN_API int mn_axpy_rms_filter_rows(float* x, int64_t ldx, const float* y, int64_t ldy, float mult, const uint16_t* w, float eps,
+                                   const uint16_t* taps_w, int taps, float* state, const int32_t* row_seq, const int32_t* row_slot,
+                                   float* h, int64_t ldh, int M, int n, void* stream);
+/* Rotary frequencies of the pairs (i, i + dims / 2), i < dims / 2: base^(-2i / dims), with YaRN interpolation when factor > 0
+ * (ramp between the dimensions whose wavelengths make `fast` and `slow` turns over `original` positions).  HOST output freq
+ * [dims / 2]; returns the factor cos and sin are multiplied by through *mag. */
+MN_API int mn_rotary_frequencies_host(int dims, double base, double factor, double original, double fast, double slow, float* freq,
+                                      float* mag);
+/* Per row and head vector of qkv fp32 [M, (H + G) * dim + G * vdim]: rotate the first rot_dims values of every q and k head at
+ * position row_slot[m] (freq device fp32 [rot_dims / 2], cos / sin times mag; rot_dims 0: none), divide q and k heads by their root
+ * mean square (unit = 0: skip), write q * q_scale to q_out [M, H * dim] and append k / v to the arenas
+ * k_arena [n_seq, t_max, G * dim], v_arena [n_seq, t_max, G * vdim] at (row_seq[m], row_slot[m]).  dim, vdim <= 512. */
+MN_API int mn_rope_unit_append(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, int rot_dims, const float* freq,
+                               float mag, int unit, float eps, float q_scale, const int32_t* row_seq, const int32_t* row_slot, float* q_out,
+                               int64_t ldq, float* k_arena, float* v_arena, int t_max, void* stream);
+/* Mean key / value of every block of `pool` slots that a row of this call completes (row_slot % pool == pool - 1):
+ * pk [n_seq, n_pool_max, G * dim], pv [n_seq, n_pool_max, G * vdim], block b of a sequence = its slots [b pool, (b + 1) pool). */
+MN_API int mn_pool_blocks_update(const float* k_arena, const float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool,
+                                 int Gd, int Gv, const int32_t* row_seq, const int32_t* row_slot, int M, void* stream);
+/* Softmax attention of q fp32 [M, H, dim] (scale included) for row m at position i = row_slot[m] of sequence row_seq[m] over the
+ * slots j with 0 <= i - j < window (window 0: every j <= i) and, with pool > 0, over the block means b with (b + 1) pool - 1 <=
+ * i - window, all in one softmax; query head h uses key / value head h / (H / G).  out[m, h * vdim + c] = out_scale * result
+ * (fp32, row stride ldo; out16: optional bf16 copy).  (H / G) * vdim <= 8 * 256 per 8 heads; any dim. */
+MN_API int mn_window_pool_attn(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk, const float* pv,
+                               const int32_t* row_seq, const int32_t* row_slot, int M, int H, int G, int dim, int vdim, int t_max,
+                               int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                               int64_t ldo16, void* stream);
+/* minGRU over each sequence's rows: z = sigmoid(zx[m, c]), u = zx[m, n + c] (biases already added), candidate = u + 1/2 (u >= 0) or
+ * sigmoid(u); S = (1 - z) S + z candidate from state fp32 [n_seq, n] (a row at slot 0 starts from zero), which is left at the
+ * sequence's last row; out[m, c] = out_scale * S * silu(g[m, c]).  Rows of one sequence are consecutive (row_back as in 9). */
+MN_API int mn_mingru_rows(const float* zx, int64_t ldzx, const float* g, int64_t ldg, float* state, const int32_t* row_seq,
+                          const int32_t* row_slot, const int32_t* row_back, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                          int64_t ldo16, int M, int n, void* stream);
+/* The `top` largest of logits[m, 0 .. E) (ties: the lower index) and the softmax over those alone: idx int32 [M, top], w fp32 [M, top] */
+MN_API int mn_router_topk_rows(const float* logits, int64_t ld, int M, int E, int top, int32_t* idx, float* w, void* stream);
+/* y[m, c] = silu(x[m, c]) * x[m, n + c]; y16: optional bf16 copy */
+MN_API int mn_silu_mul_rows(const float* x, int64_t ldx, float* y, int64_t ldy, uint16_t* y16, int64_t ldy16, int M, int n, void* stream);
+/* C[z] fp32 [N] = A[z / a_div] . W[w_idx[z]]^T for z < Z: one input row against the weight block its index names (fp32 FMA; A row
+ * stride lda, weight block stride w_bs, C row stride ldc). */
+MN_API int mn_gemv_f32_indexed(const float* A, int64_t lda, int a_div, const uint16_t* W, int64_t ldw, int64_t w_bs, const int32_t* w_idx,
+                               float* C, int64_t ldc, int Z, int N, int K, void* stream);
+/* x[m] += mult * (sum_j w[m, j] y[r(m, j)] + sigmoid(sg[m * ldsg]) * shared[m]) with r(m, j) = slot_of ? slot_of[m * top + j] :
+ * m * top + j; shared / sg may be NULL */
+MN_API int mn_moe_combine_residual(float* x, int64_t ldx, const float* y, int64_t ldy, const int32_t* slot_of, const float* w, int top,
+                                   const float* shared, int64_t lds, const float* sg, int64_t ldsg, float mult, int M, int n, void* stream);
+
+typedef struct mn_pmix_layer {
+  int32_t heads, kv_heads, dim, vdim;
+  int32_t conv;                                    /* taps of the q / k / v filter, 0: none */
+  int32_t rot_dims;                                /* 0: no rotation */
+  int32_t unit_qk;                                 /* 1: q and k heads divided by their root mean square */
+  int32_t window, pool;                            /* 0, 0: every earlier token */
+  int32_t gru;                                     /* width of the recurrence */
+  int32_t experts, top, ff, shared_ff;             /* experts 0: the layer has no feed-forward; shared_ff 0: no shared expert */
+  float scale, rot_mag, left_scale, right_scale;
+  const float* rot_freq;                           /* DEVICE fp32 [rot_dims / 2] */
+  const uint16_t *norm1, *norm2;                   /* [width] */
+  const uint16_t *canon1, *canon2;                 /* [width, taps] (model.taps 0: unused) */
+  const uint16_t *w_in, *b_in;                     /* [q ; k ; v ; z ; x ; g] rows, bias (zero outside z and x) */
+  const uint16_t *w_conv;                          /* [(heads + kv_heads) * dim + kv_heads * vdim, conv] */
+  const uint16_t *w_out;                           /* [width, heads * vdim + gru] = [left o | right o] */
+  const uint16_t *w_ff_in, *b_ff_in;               /* [shared gate ; shared up ; router ; shared gate logit] rows, bias (router's) */
+  const uint16_t *w_shared_down;                   /* [width, shared_ff] */
+  const uint16_t *w_gate_up;                       /* [experts, 2 ff, width] */
+  const uint16_t *w_down;                          /* [experts, width, ff] */
+} mn_pmix_layer;
+typedef struct mn_pmix_model {
+  int32_t width, n_layers, n_runs, taps, arith;    /* taps: of the sublayer-input filter, 0: none */
+  float eps, mult;
+  const mn_pmix_layer* layers;                     /* HOST array [n_layers] */
+  const int32_t* run_layer;                        /* HOST [n_runs]: the layer of every run */
+  const uint8_t* run_readd;                        /* HOST [n_runs]: 1 = the step's input rows are added to x before this run */
+  const uint16_t* final_w;
+} mn_pmix_model;
+typedef struct mn_pmix_state {                     /* HOST arrays [n_runs] of device pointers, fp32 */
+  float* const* k;                                 /* [n_seq, t_max, kv_heads * dim] */
+  float* const* v;                                 /* [n_seq, t_max, kv_heads * vdim] */
+  float* const* pk;                                /* [n_seq, n_pool_max, kv_heads * dim]  (pool 0: unused) */
+  float* const* pv;
+  float* const* canon;                             /* [2, n_seq, taps - 1, width]: mixer, feed-forward */
+  float* const* conv;                              /* [n_seq, conv - 1, q + k + v channels] */
+  float* const* gru;                               /* [n_seq, gru] */
+  int32_t n_seq, t_max, n_pool_max;
+} mn_pmix_state;
+MN_API size_t mn_sizeof_pmix_layer(void);
+MN_API size_t mn_sizeof_pmix_model(void);
+MN_API size_t mn_sizeof_pmix_state(void);
+/* One pass of the stack over M rows; rows, row arrays, out and trace as mn_seq_step (trace: fp32 [n_runs, M, width]).
+ * flags: MN_SEQ_ROWS_DISTINCT fuses the residual add / norm / filter launches of decode rows. */
+MN_API size_t mn_pmix_workspace_bytes(const mn_pmix_model* m, int M);
+MN_API int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
+                        const int32_t* row_slot, const int32_t* row_back, int flags, float* out, float* trace, void* workspace,
+                        size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

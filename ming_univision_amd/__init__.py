@@ -12,10 +12,11 @@ import os as _os
 # queues unless told otherwise (4 groups: 1447 vs 1686 tokens/s).  Only effective if HIP has not initialised yet.
 _os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
 
-from .configuration import BailingMoeConfig, MingTokConfig, MingUniVisionConfig, PizitarConfig  # noqa: F401,E402
+from .configuration import BailingMoeConfig, MingTokConfig, MingUniVisionConfig, PizitarConfig, SakinexConfig  # noqa: F401,E402
 
 __all__ = ["BailingMoeConfig", "MingTokConfig", "MingUniVisionConfig", "MingTok", "MingUniVisionInfer",
-           "MingUniVisionForConditionalGeneration", "BailingMMProcessor", "PizitarConfig", "PizitarDecoder", "PizitarForCausalLM", "load_model"]
+           "MingUniVisionForConditionalGeneration", "BailingMMProcessor", "PizitarConfig", "PizitarDecoder", "PizitarForCausalLM", "SakinexConfig",
+           "SakinexDecoder", "SakinexForCausalLM", "load_model"]
 
 
 def __getattr__(name):  # lazy: keep `import ming_univision_amd` cheap and torch-free
@@ -34,6 +35,9 @@ def __getattr__(name):  # lazy: keep `import ming_univision_amd` cheap and torch
     if name in ("PizitarDecoder", "PizitarForCausalLM"):
         from . import pizitar
         return getattr(pizitar, name)
+    if name in ("SakinexDecoder", "SakinexForCausalLM"):
+        from . import sakinex
+        return getattr(sakinex, name)
     if name == "load_model":
         from .infer import load_model
         return load_model

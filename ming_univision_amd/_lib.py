@@ -124,10 +124,30 @@ class SeqState(C.Structure):
     _fields_ = [("latent", PP), ("taps", C.c_void_p), ("n_seq", C.c_int32), ("t_max", C.c_int32)]
 
 
+class PmixLayer(C.Structure):
+    _fields_ = [(k, C.c_int32) for k in ("heads", "kv_heads", "dim", "vdim", "conv", "rot_dims", "unit_qk", "window", "pool", "gru",
+                                         "experts", "top", "ff", "shared_ff")] + \
+               [(k, C.c_float) for k in ("scale", "rot_mag", "left_scale", "right_scale")] + \
+               [(k, C.c_void_p) for k in ("rot_freq", "norm1", "norm2", "canon1", "canon2", "w_in", "b_in", "w_conv", "w_out", "w_ff_in",
+                                          "b_ff_in", "w_shared_down", "w_gate_up", "w_down")]
+
+
+class PmixModel(C.Structure):
+    _fields_ = [("width", C.c_int32), ("n_layers", C.c_int32), ("n_runs", C.c_int32), ("taps", C.c_int32), ("arith", C.c_int32),
+                ("eps", C.c_float), ("mult", C.c_float), ("layers", C.POINTER(PmixLayer)), ("run_layer", C.POINTER(C.c_int32)),
+                ("run_readd", C.POINTER(C.c_uint8)), ("final_w", C.c_void_p)]
+
+
+class PmixState(C.Structure):
+    _fields_ = [(k, PP) for k in ("k", "v", "pk", "pv", "canon", "conv", "gru")] + \
+               [("n_seq", C.c_int32), ("t_max", C.c_int32), ("n_pool_max", C.c_int32)]
+
+
 # (struct id of mn_struct_layout, its mn_sizeof_* export, the ctypes mirror): checked against the library at load time (`lib()`)
 STRUCTS = ((0, "mn_sizeof_skinny_args", SkinnyArgs), (1, "mn_sizeof_rf_head", RfHead), (2, "mn_sizeof_llm", Llm),
            (3, "mn_sizeof_semdec", SemDec), (4, "mn_sizeof_tp_comm", TpComm), (5, "mn_sizeof_llm_tp", LlmTp),
-           (6, "mn_sizeof_seq_layer", SeqLayer), (7, "mn_sizeof_seq_model", SeqModel), (8, "mn_sizeof_seq_state", SeqState))
+           (6, "mn_sizeof_seq_layer", SeqLayer), (7, "mn_sizeof_seq_model", SeqModel), (8, "mn_sizeof_seq_state", SeqState),
+           (9, "mn_sizeof_pmix_layer", PmixLayer), (10, "mn_sizeof_pmix_model", PmixModel), (11, "mn_sizeof_pmix_state", PmixState))
 
 
 def check_struct_layouts(handle):
@@ -286,6 +306,23 @@ SYMBOLS = {
     "mn_seq_step": (_i, [C.POINTER(SeqModel), C.POINTER(SeqState), _p, _i64, _i, _p, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
     "mn_gated_norm_filter_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _f, _p, _i64, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "mn_seq_logits": (_i, [_p, _i64, _i, _p, _i, _i, _f, _i, _p, _i64, _p, _sz, _p]),
+    # section 10: parallel-mixer sequence models
+    "mn_sizeof_pmix_layer": (_sz, []), "mn_sizeof_pmix_model": (_sz, []), "mn_sizeof_pmix_state": (_sz, []),
+    "mn_tap_conv_rows": (_i, [_p, _i64, _p, _i, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
+    "mn_axpy_rms_rows": (_i, [_p, _i64, _p, _i64, _f, _p, _f, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_axpy_rms_filter_rows": (_i, [_p, _i64, _p, _i64, _f, _p, _f, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _p]),
+    "mn_rotary_frequencies_host": (_i, [_i, C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.POINTER(C.c_float),
+                                        C.POINTER(C.c_float)]),
+    "mn_rope_unit_append": (_i, [_p, _i64, _i, _i, _i, _i, _i, _i, _p, _f, _i, _f, _f, _p, _p, _p, _i64, _p, _p, _i, _p]),
+    "mn_pool_blocks_update": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p]),
+    "mn_window_pool_attn": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64, _p]),
+    "mn_mingru_rows": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _f, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_router_topk_rows": (_i, [_p, _i64, _i, _i, _i, _p, _p, _p]),
+    "mn_silu_mul_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_gemv_f32_indexed": (_i, [_p, _i64, _i, _p, _i64, _i64, _p, _p, _i64, _i, _i, _i, _p]),
+    "mn_moe_combine_residual": (_i, [_p, _i64, _p, _i64, _p, _p, _i, _p, _i64, _p, _i64, _f, _i, _i, _p]),
+    "mn_pmix_workspace_bytes": (_sz, [C.POINTER(PmixModel), _i]),
+    "mn_pmix_step": (_i, [C.POINTER(PmixModel), C.POINTER(PmixState), _p, _i64, _i, _p, _p, _p, _i, _p, _p, _p, _sz, _p]),
     "mn_semdec_step": (_i, [C.POINTER(SemDec), _p, _i, _p, _p, _p, _p, _i, _i64, _p, _p, _p, _sz, _p]),
 }
 
@@ -306,7 +343,7 @@ def lib():
         fn = getattr(handle, name)  # AttributeError if the symbol is missing
         fn.restype = res
         fn.argtypes = args
-    if handle.mn_version() < 126:
+    if handle.mn_version() < 127:
         raise RuntimeError("libmingnative.so is too old")
     check_struct_layouts(handle)
     _lib = handle

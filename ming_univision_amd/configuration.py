@@ -5,6 +5,8 @@
   MingUniVisionConfig  <- mingunivision/configuration_bailingmm.py:20-31
                           (+ `vishead_diffloss_config`, asserted at modeling_bailingmm.py:118)
 
+  SakinexConfig        <- a decoder-only language model of parallel-mixer layers (windowed attention beside a minGRU, mixture-of-
+                          experts feed-forward; no reference counterpart)
   PizitarConfig        <- a decoder-only language model of latent-attention layers (no reference counterpart): config.json keys
                           `architecture`, `width`, `vocab`, `layers`, `canon.taps`, `norm.eps`, `logit_softcap`
 
@@ -376,16 +378,134 @@ def pizitar_param_shapes(cfg: PizitarConfig):
     return s
 
 
+# ---- Sakinex ---------------------------------------------------------------------------------------------------------------
+SAKINEX_MIXERS = ("parallel",)
+
+
+class SakinexConfig(_Config):
+    """A stack of parallel-mixer layers.  `layers` is a list of dicts(type, mixer, mlp):
+    type  "parallel": a windowed attention (`mixer.left`) beside a minGRU (`mixer.right`), summed with `left_scale` / `right_scale`
+    left  heads, kv_heads, dim (query / key size per head), vdim, scale (of the scores); optional conv (taps of the filter on the
+          projected q / k / v channels), rot dict(base, dims, optional scaling dict(factor, original, fast, slow)), mask
+          dict(size = window, optional pool = tokens per pooled block before the window); no mask: every earlier token
+    right width
+    mlp   None or dict(kind="moe", router dict(experts, top), expert dict(ff), optional shared dict(ff))
+    canon dict(taps): the causal filter added to what every sublayer reads (absent: none); loop dict(start, stop, times): layers
+    start .. stop - 1 run `times` times in a row with the same weights.  Every size is read from here or from the tensors; nothing
+    is assumed equal between layers."""
+    model_type = "sakinex"
+
+    def __init__(self, width=256, vocab=1024, layers=(), canon=None, norm=None, loop=None, residual_mult=1.0, architecture="Sakinex",
+                 **kwargs):
+        self.architecture = architecture
+        self.width, self.vocab = int(width), int(vocab)
+        self.layers = [copy.deepcopy(dict(ly)) for ly in layers]
+        self.canon = dict(canon) if canon else None
+        self.norm = dict(norm or {"eps": 1e-6})
+        self.loop = dict(loop) if loop else None
+        self.residual_mult = float(residual_mult)
+        super().__init__(**kwargs)
+        self.validate()
+
+    taps = property(lambda self: int(self.canon["taps"]) if self.canon else 0)
+    eps = property(lambda self: float(self.norm["eps"]))
+
+    def runs(self):
+        """[(layer, add the embedding rows first)] in execution order."""
+        n = len(self.layers)
+        if not self.loop:
+            return [(i, False) for i in range(n)]
+        a, b, times = int(self.loop["start"]), int(self.loop["stop"]), int(self.loop["times"])
+        out = [(i, False) for i in range(a)]
+        for r in range(times):
+            out += [(i, r > 0 and i == a) for i in range(a, b)]
+        return out + [(i, False) for i in range(b, n)]
+
+    def validate(self):
+        if self.canon and self.taps < 1:
+            raise ValueError("canon.taps must be >= 1")
+        if self.loop:
+            a, b, times = (int(self.loop[k]) for k in ("start", "stop", "times"))
+            if not (0 <= a <= b <= len(self.layers)) or times < 1:
+                raise ValueError(f"loop {self.loop}: 0 <= start <= stop <= {len(self.layers)} layers and times >= 1")
+        for i, ly in enumerate(self.layers):
+            if ly.get("type") not in SAKINEX_MIXERS:
+                raise ValueError(f"layer {i}: unknown mixer type {ly.get('type')!r} (known: {SAKINEX_MIXERS})")
+            m = ly["mixer"]
+            for k in ("left", "right", "left_scale", "right_scale"):
+                if k not in m:
+                    raise ValueError(f"layer {i}: mixer lacks {k!r}")
+            L = m["left"]
+            for k in ("heads", "kv_heads", "dim", "vdim", "scale"):
+                if k not in L:
+                    raise ValueError(f"layer {i}: mixer.left lacks {k!r}")
+            if L["heads"] % L["kv_heads"]:
+                raise ValueError(f"layer {i}: {L['heads']} query heads do not divide over {L['kv_heads']} key/value heads")
+            rot = L.get("rot")
+            if rot and (rot["dims"] % 2 or rot["dims"] > L["dim"]):
+                raise ValueError(f"layer {i}: rot.dims = {rot['dims']} must be even and at most dim = {L['dim']}")
+            mask = L.get("mask")
+            if mask and (int(mask["size"]) < 1 or int(mask.get("pool") or 1) < 1):
+                raise ValueError(f"layer {i}: mask {mask}: size >= 1, pool >= 1")
+            if "width" not in m["right"]:
+                raise ValueError(f"layer {i}: mixer.right lacks 'width'")
+            mlp = ly.get("mlp")
+            if mlp is not None:
+                if mlp.get("kind") != "moe":
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+                if not (1 <= int(mlp["router"]["top"]) <= int(mlp["router"]["experts"])):
+                    raise ValueError(f"layer {i}: router {mlp['router']}: 1 <= top <= experts")
+
+
+def sakinex_param_shapes(cfg: SakinexConfig):
+    """{tensor name: shape} of a Sakinex checkpoint (`l<i>.` per layer; `.b` = the bias and `.conv` the filter of the tensor it follows)."""
+    W, V, taps = cfg.width, cfg.vocab, cfg.taps
+    s = {"embed": (V, W)}
+    for i, ly in enumerate(cfg.layers):
+        p, m, mlp = f"l{i}.", ly["mixer"], ly.get("mlp")
+        L, wr = m["left"], int(m["right"]["width"])
+        H, G, d, e = int(L["heads"]), int(L["kv_heads"]), int(L["dim"]), int(L["vdim"])
+        s[p + "norm1"] = (W,)
+        for n, rows in (("q", H * d), ("k", G * d), ("v", G * e)):
+            s[p + "mix.left." + n] = (rows, W)
+            if L.get("conv"):
+                s[p + "mix.left." + n + ".conv"] = (rows, int(L["conv"]))
+        s[p + "mix.left.o"] = (W, H * e)
+        for n in ("z", "x"):
+            s[p + "mix.right." + n], s[p + "mix.right." + n + ".b"] = (wr, W), (wr,)
+        s[p + "mix.right.g"], s[p + "mix.right.o"] = (wr, W), (W, wr)
+        if taps:
+            s[p + "canon1"] = (W, taps)
+        if mlp is not None:
+            s[p + "norm2"] = (W,)
+            E, ff = int(mlp["router"]["experts"]), int(mlp["expert"]["ff"])
+            for j in range(E):
+                s[f"{p}mlp.e{j}.gate"], s[f"{p}mlp.e{j}.up"], s[f"{p}mlp.e{j}.down"] = (ff, W), (ff, W), (W, ff)
+            s[p + "mlp.router"], s[p + "mlp.router.b"] = (E, W), (E,)
+            if mlp.get("shared"):
+                fs = int(mlp["shared"]["ff"])
+                s[p + "mlp.shared.gate"], s[p + "mlp.shared.up"], s[p + "mlp.shared.down"] = (fs, W), (fs, W), (W, fs)
+                s[p + "mlp.shared.sg"] = (1, W)
+            if taps:
+                s[p + "canon2"] = (W, taps)
+    s["final.norm"], s["head"] = (W,), (V, W)
+    return s
+
+
 # ---- registry: which configuration class a config.json belongs to -------------------------------------------------------------
 def _is_pizitar(d):
     return d.get("architecture") == "Pizitar" or d.get("model_type") == "pizitar"
+
+
+def _is_sakinex(d):
+    return d.get("architecture") == "Sakinex" or d.get("model_type") == "sakinex"
 
 
 def _is_ming_univision(d):
     return "llm_config" in d or d.get("model_type") in ("bailingmm", "ming_univision")
 
 
-MODEL_REGISTRY = [("pizitar", _is_pizitar, PizitarConfig), ("ming_univision", _is_ming_univision, MingUniVisionConfig)]
+MODEL_REGISTRY = [("pizitar", _is_pizitar, PizitarConfig), ("sakinex", _is_sakinex, SakinexConfig), ("ming_univision", _is_ming_univision, MingUniVisionConfig)]
 
 
 def config_from_pretrained(path):

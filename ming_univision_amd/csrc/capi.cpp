@@ -129,12 +129,30 @@ extern "C" int mn_struct_layout(int which, size_t* offsets, int cap) {
       F(latent) F(taps) F(n_seq) F(t_max)
 #undef F
   };
-  const size_t* tab[] = {skinny, rf, llm, semdec, comm, llm_tp, seq_layer, seq_model, seq_state};
+  static const size_t pmix_layer[] = {
+#define F(f) MN_OFF(mn_pmix_layer, f)
+      F(heads) F(kv_heads) F(dim) F(vdim) F(conv) F(rot_dims) F(unit_qk) F(window) F(pool) F(gru) F(experts) F(top) F(ff) F(shared_ff)
+      F(scale) F(rot_mag) F(left_scale) F(right_scale) F(rot_freq) F(norm1) F(norm2) F(canon1) F(canon2) F(w_in) F(b_in) F(w_conv) F(w_out)
+      F(w_ff_in) F(b_ff_in) F(w_shared_down) F(w_gate_up) F(w_down)
+#undef F
+  };
+  static const size_t pmix_model[] = {
+#define F(f) MN_OFF(mn_pmix_model, f)
+      F(width) F(n_layers) F(n_runs) F(taps) F(arith) F(eps) F(mult) F(layers) F(run_layer) F(run_readd) F(final_w)
+#undef F
+  };
+  static const size_t pmix_state[] = {
+#define F(f) MN_OFF(mn_pmix_state, f)
+      F(k) F(v) F(pk) F(pv) F(canon) F(conv) F(gru) F(n_seq) F(t_max) F(n_pool_max)
+#undef F
+  };
+  const size_t* tab[] = {skinny, rf, llm, semdec, comm, llm_tp, seq_layer, seq_model, seq_state, pmix_layer, pmix_model, pmix_state};
   const int cnt[] = {(int)(sizeof(skinny) / sizeof(size_t)), (int)(sizeof(rf) / sizeof(size_t)), (int)(sizeof(llm) / sizeof(size_t)),
                      (int)(sizeof(semdec) / sizeof(size_t)), (int)(sizeof(comm) / sizeof(size_t)), (int)(sizeof(llm_tp) / sizeof(size_t)),
                      (int)(sizeof(seq_layer) / sizeof(size_t)), (int)(sizeof(seq_model) / sizeof(size_t)),
-                     (int)(sizeof(seq_state) / sizeof(size_t))};
-  MN_CHECK_ARG(which >= 0 && which < 9, "mn_struct_layout: unknown struct id");
+                     (int)(sizeof(seq_state) / sizeof(size_t)), (int)(sizeof(pmix_layer) / sizeof(size_t)),
+                     (int)(sizeof(pmix_model) / sizeof(size_t)), (int)(sizeof(pmix_state) / sizeof(size_t))};
+  MN_CHECK_ARG(which >= 0 && which < 12, "mn_struct_layout: unknown struct id");
   for (int i = 0; i < cnt[which] && i < cap; ++i) offsets[i] = tab[which][i];
   return cnt[which];
 }

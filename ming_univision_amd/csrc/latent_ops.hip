@@ -193,12 +193,13 @@ bool launch_row_block(const RowArgs& a, int M, hipStream_t st) {
 __global__ __launch_bounds__(256) void tap_filter_kernel(const float* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int taps,
                                                          const float* __restrict__ state, const int32_t* __restrict__ row_seq,
                                                          const int32_t* __restrict__ row_slot, const int32_t* __restrict__ row_back,
-                                                         float* __restrict__ y, int64_t ldy, bf16_t* __restrict__ y16, int64_t ldy16, int n) {
+                                                         float* __restrict__ y, int64_t ldy, bf16_t* __restrict__ y16, int64_t ldy16, int n,
+                                                         float self_w) {
   const int m = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
   if (c >= n) return;
   const int seq = row_seq[m], slot = row_slot[m], back = row_back[m];
   const float cur = x[(int64_t)m * ldx + c];
-  float acc = cur;
+  float acc = self_w * cur;                         // 1: the input is added to its filter, 0: the filter alone
   for (int k = 0; k < taps; ++k) {
     float v = 0.f;
     if (k <= back) v = x[(int64_t)(m - k) * ldx + c];
@@ -758,8 +759,18 @@ extern "C" int mn_tap_filter_rows(const float* x, int64_t ldx, const uint16_t* w
                "mn_tap_filter_rows: bad args");
   MN_CHECK_ARG(M <= 65535, "mn_tap_filter_rows: at most 65535 rows per call");
   hipLaunchKernelGGL(tap_filter_kernel, dim3((unsigned)mn_cdiv(n, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), x, ldx, w, taps, state,
-                     row_seq, row_slot, row_back, y, ldy, y16, ldy16, n);
+                     row_seq, row_slot, row_back, y, ldy, y16, ldy16, n, 1.0f);
   MN_CHECK_LAUNCH("mn_tap_filter_rows");
+  return MN_OK;
+}
+
+extern "C" int mn_tap_conv_rows(const float* x, int64_t ldx, const uint16_t* w, int taps, const float* state, const int32_t* row_seq,
+                                const int32_t* row_slot, const int32_t* row_back, float* y, int64_t ldy, int M, int n, void* stream) {
+  MN_CHECK_ARG(x && w && taps >= 1 && (state || taps == 1) && row_seq && row_slot && row_back && y && M >= 1 && M <= 65535 && n >= 1,
+               "mn_tap_conv_rows: bad args");
+  hipLaunchKernelGGL(tap_filter_kernel, dim3((unsigned)mn_cdiv(n, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), x, ldx, w, taps, state,
+                     row_seq, row_slot, row_back, y, ldy, (bf16_t*)nullptr, (int64_t)0, n, 0.0f);
+  MN_CHECK_LAUNCH("mn_tap_conv_rows");
   return MN_OK;
 }
 

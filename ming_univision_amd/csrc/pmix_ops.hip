@@ -1,0 +1,554 @@
+// pmix_ops.hip — row operators of parallel-mixer sequence models (mingnative.h section 10): a windowed softmax attention with
+// pooled far blocks beside a minGRU recurrence, RMS pre-norms, a mixture-of-experts feed-forward.  Everything works on fp32 rows
+// [M, n] of a step (tokens of one or several cache sequences, each sequence's rows consecutive) and bf16 weights; every size and
+// constant is an argument.
+//
+//   mn_axpy_rms_rows           x += mult * y;  n = x / sqrt(mean(x^2) + eps) * w
+//   mn_axpy_rms_filter_rows    the same for decode rows, with the sublayer-input filter and its state update in the launch
+//   mn_rope_unit_append        rotary (frequency table) + unit-RMS per head on q and k, q scaled, k / v appended to their arenas
+//   mn_pool_blocks_update      mean key / value of the blocks a step completes
+//   mn_window_pool_attn        softmax over the window's tokens and the block means before it, online softmax in fp32
+//   mn_mingru_rows             S = (1 - z) S + z c over each sequence's rows, gated output
+//   mn_router_topk_rows        top-k of the router logits, softmax over the chosen
+//   mn_silu_mul_rows           silu(gate) * up
+//   mn_gemv_f32_indexed        one row against the weight block an index names (experts of few rows, and the fp32 path)
+//   mn_moe_combine_residual    x += mult * (sum_j w_j y_j + sigmoid(sg) shared)
+#include <math.h>
+
+#include "common.h"
+
+extern "C" int mn_rotary_frequencies_host(int dims, double base, double factor, double original, double fast, double slow, float* freq,
+                                          float* mag) {
+  MN_CHECK_ARG(dims >= 2 && (dims % 2) == 0 && base > 1.0 && freq && mag, "mn_rotary_frequencies_host: bad args (dims=%d)", dims);
+  const int half = dims / 2;
+  const double two_pi = 6.283185307179586476925286766559;
+  double lo = 0, hi = 0;
+  if (factor > 0) {
+    MN_CHECK_ARG(original > 0 && fast > 0 && slow > 0, "mn_rotary_frequencies_host: bad scaling");
+    auto dim_of = [&](double turns) { return dims * log(original / (two_pi * turns)) / (2.0 * log(base)); };
+    lo = floor(dim_of(fast)); if (lo < 0) lo = 0;
+    hi = ceil(dim_of(slow)); if (hi > dims - 1) hi = dims - 1;
+  }
+  for (int i = 0; i < half; ++i) {
+    const double f = pow(base, -2.0 * i / dims);
+    double v = f;
+    if (factor > 0) {
+      double den = hi - lo; if (den < 0.001) den = 0.001;
+      double ramp = (i - lo) / den; if (ramp < 0) ramp = 0; if (ramp > 1) ramp = 1;
+      v = f / factor * ramp + f * (1.0 - ramp);
+    }
+    freq[i] = (float)v;
+  }
+  *mag = factor > 0 ? (float)(0.1 * log(factor) + 1.0) : 1.0f;
+  return MN_OK;
+}
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// one wave per row: x += mult * y, then RMS norm with a weight
+__global__ __launch_bounds__(256) void axpy_rms_kernel(float* __restrict__ x, int64_t ldx, const float* __restrict__ y, int64_t ldy,
+                                                       float mult, const bf16_t* __restrict__ w, float eps, float* __restrict__ nout,
+                                                       int64_t ldn, bf16_t* __restrict__ n16, int64_t ldn16, int M, int n) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= M) return;
+  float* xr = x + (int64_t)row * ldx;
+  float s = 0.f;
+  for (int i = lane; i < n; i += 64) {
+    float v = xr[i];
+    if (y) { v += mult * y[(int64_t)row * ldy + i]; xr[i] = v; }
+    s += v * v;
+  }
+  if (!nout && !n16) return;
+  const float r = 1.0f / sqrtf(wave_sum(s) / (float)n + eps);
+  for (int i = lane; i < n; i += 64) {
+    const float o = xr[i] * r * bf16_to_f32(w[i]);
+    if (nout) nout[(int64_t)row * ldn + i] = o;
+    if (n16) n16[(int64_t)row * ldn16 + i] = f32_to_bf16(o);
+  }
+}
+
+// Decode rows, one workgroup per row, the row in registers: x += mult * y; n = RMS(x) w; h = n + filter(n, state); state moves on.
+constexpr int FUSED_MAX_TAPS = 8;
+struct AxpyRmsFilterArgs {
+  float* x; int64_t ldx;
+  const float* y; int64_t ldy; float mult;
+  const bf16_t* w; float eps;
+  const bf16_t* taps_w; int taps;
+  float* state; const int32_t* row_seq; const int32_t* row_slot;
+  float* h; int64_t ldh;
+  int n;
+};
+
+template <int VPT>
+__global__ __launch_bounds__(256) void axpy_rms_filter_kernel(AxpyRmsFilterArgs a) {
+  __shared__ float red[8];
+  const int row = blockIdx.x, tid = threadIdx.x, n = a.n;
+  const bool filter = a.taps_w != nullptr && a.taps >= 1;
+  const int seq = filter ? a.row_seq[row] : 0, slot = filter ? a.row_slot[row] : 0;
+  float* const st0 = (filter && a.taps > 1) ? a.state + (int64_t)seq * (a.taps - 1) * n : nullptr;
+  float xv[VPT], sv[VPT][FUSED_MAX_TAPS - 1];
+  // every load of the row is issued before the first store
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = tid + 256 * i, cc = c < n ? c : 0;
+    float t = a.x[(int64_t)row * a.ldx + cc];
+    if (a.y) t += a.mult * a.y[(int64_t)row * a.ldy + cc];
+    xv[i] = c < n ? t : 0.f;
+#pragma unroll
+    for (int k = 1; k < FUSED_MAX_TAPS; ++k) sv[i][k - 1] = (st0 && k < a.taps) ? st0[(int64_t)(k - 1) * n + cc] : 0.f;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) s += xv[i] * xv[i];
+  const float r = 1.0f / sqrtf(block_sum(s, red) / (float)n + a.eps);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = tid + 256 * i;
+    if (c >= n) continue;
+    if (a.y) a.x[(int64_t)row * a.ldx + c] = xv[i];
+    const float nv = xv[i] * r * bf16_to_f32(a.w[c]);
+    float acc = nv;
+    if (filter) {
+      const bf16_t* tw = a.taps_w + (int64_t)c * a.taps;
+      acc += bf16_to_f32(tw[a.taps - 1]) * nv;
+#pragma unroll
+      for (int k = 1; k < FUSED_MAX_TAPS; ++k)
+        if (k < a.taps && slot - k >= 0) acc += bf16_to_f32(tw[a.taps - 1 - k]) * sv[i][k - 1];
+      if (st0) {
+        float* st = st0 + c;
+#pragma unroll
+        for (int k = FUSED_MAX_TAPS - 2; k >= 1; --k)
+          if (k < a.taps - 1) st[(int64_t)k * n] = sv[i][k - 1];
+        st[0] = nv;
+      }
+    }
+    a.h[(int64_t)row * a.ldh + c] = acc;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// One wave per (row, head vector): q heads 0 .. H - 1, k heads H .. H + G - 1, v heads after them.  A lane holds the pairs
+// (i, i + half) for i = lane, lane + 64, ... and the values past rot_dims: at most 8 of each (dim <= 512).
+struct RopeArgs {
+  const float* qkv; int64_t ldqkv;
+  int H, G, dim, vdim, rot_dims;
+  const float* freq; float mag; int unit; float eps, q_scale;
+  const int32_t* row_seq; const int32_t* row_slot;
+  float* q_out; int64_t ldq;
+  float* k_arena; float* v_arena; int t_max;
+};
+
+__global__ __launch_bounds__(256) void rope_unit_append_kernel(RopeArgs a, int M) {
+  const int hv = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, m = blockIdx.y;
+  const int nh = a.H + 2 * a.G;
+  if (hv >= nh) return;
+  const float* src = a.qkv + (int64_t)m * a.ldqkv;
+  const int64_t crow = (int64_t)a.row_seq[m] * a.t_max + a.row_slot[m];
+  if (hv >= a.H + a.G) {                                         // a value head: copied into its arena
+    const int g = hv - a.H - a.G;
+    src += (int64_t)(a.H + a.G) * a.dim + (int64_t)g * a.vdim;
+    float* dst = a.v_arena + crow * ((int64_t)a.G * a.vdim) + (int64_t)g * a.vdim;
+    for (int i = lane; i < a.vdim; i += 64) dst[i] = src[i];
+    return;
+  }
+  const bool is_q = hv < a.H;
+  src += (int64_t)hv * a.dim;
+  float* dst = is_q ? a.q_out + (int64_t)m * a.ldq + (int64_t)hv * a.dim
+                    : a.k_arena + crow * ((int64_t)a.G * a.dim) + (int64_t)(hv - a.H) * a.dim;
+  const int half = a.rot_dims / 2;
+  const float pos = (float)a.row_slot[m];
+  float lo[4], hi[4], rest[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + 64 * j;
+    lo[j] = hi[j] = 0.f;
+    if (i < half) {
+      const float u = src[i], v = src[i + half];
+      const float ang = pos * a.freq[i];
+      const float c = cosf(ang) * a.mag, s = sinf(ang) * a.mag;
+      lo[j] = u * c - v * s;
+      hi[j] = v * c + u * s;
+      ss += lo[j] * lo[j] + hi[j] * hi[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int i = a.rot_dims + lane + 64 * j;
+    rest[j] = 0.f;
+    if (i < a.dim) { rest[j] = src[i]; ss += rest[j] * rest[j]; }
+  }
+  float r = 1.0f;
+  if (a.unit) r = 1.0f / sqrtf(wave_sum(ss) / (float)a.dim + a.eps);
+  if (is_q) r *= a.q_scale;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + 64 * j;
+    if (i < half) { dst[i] = lo[j] * r; dst[i + half] = hi[j] * r; }
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int i = a.rot_dims + lane + 64 * j;
+    if (i < a.dim) dst[i] = rest[j] * r;
+  }
+}
+
+// grid (ceil((Gd + Gv) / 256), M): a row that completes a block writes the block's means (slots summed in ascending order)
+__global__ __launch_bounds__(256) void pool_blocks_kernel(const float* __restrict__ k_arena, const float* __restrict__ v_arena, int t_max,
+                                                          float* __restrict__ pk, float* __restrict__ pv, int n_pool_max, int pool, int Gd,
+                                                          int Gv, const int32_t* __restrict__ row_seq, const int32_t* __restrict__ row_slot) {
+  const int m = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  const int slot = row_slot[m];
+  if ((slot % pool) != pool - 1 || c >= Gd + Gv) return;
+  const int b = slot / pool, seq = row_seq[m];
+  if (b >= n_pool_max) return;
+  const bool is_k = c < Gd;
+  const int cc = is_k ? c : c - Gd, n = is_k ? Gd : Gv;
+  const float* src = (is_k ? k_arena : v_arena) + ((int64_t)seq * t_max + (int64_t)b * pool) * n + cc;
+  float s = 0.f;
+  for (int j = 0; j < pool; ++j) s += src[(int64_t)j * n];
+  (is_k ? pk : pv)[((int64_t)seq * n_pool_max + b) * n + cc] = s / (float)pool;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// Attention, plain form: one workgroup per (row, key/value head, chunk of <= 8 query heads of its group).  Keys are walked in
+// tiles of 256 (block means first, then the window's tokens): a thread scores one key for the chunk's heads, the tile's softmax
+// statistics are merged into the running ones, then the threads turn to output columns and add the tile's weighted values.
+constexpr int ATT_R = 8, ATT_TILE = 256, ATT_NOUT = 8;
+struct AttnArgs {
+  const float* q; int64_t ldq;
+  const float *k, *v, *pk, *pv;
+  const int32_t* row_seq; const int32_t* row_slot;
+  int H, G, dim, vdim, t_max, n_pool_max, window, pool;
+  float out_scale;
+  float* out; int64_t ldo; bf16_t* out16; int64_t ldo16;
+};
+
+__global__ __launch_bounds__(256) void window_pool_attn_kernel(AttnArgs a) {
+  extern __shared__ float lds[];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  const int rep = a.H / a.G, chunks = (rep + ATT_R - 1) / ATT_R;
+  const int g = blockIdx.y / chunks, h0 = g * rep + (blockIdx.y % chunks) * ATT_R;
+  const int R = min(ATT_R, g * rep + rep - h0);
+  float* qs = lds;                              // [R][dim]
+  float* sc = qs + ATT_R * a.dim;               // [R][ATT_TILE]
+  float* stat = sc + ATT_R * ATT_TILE;          // [R] running max, [R] running sum, [R] rescale of this tile
+  const int seq = a.row_seq[m], pos = a.row_slot[m];
+  int t0 = 0, nb = 0;
+  if (a.window > 0) {
+    t0 = max(0, pos - a.window + 1);
+    if (a.pool > 0 && pos - a.window + 1 >= 0) nb = (pos - a.window + 1) / a.pool;
+  }
+  const int nk = nb + (pos - t0 + 1);
+  for (int e = tid; e < R * a.dim; e += 256) qs[e] = a.q[(int64_t)m * a.ldq + (int64_t)h0 * a.dim + e];
+  if (tid < ATT_R) { stat[tid] = -INFINITY; stat[ATT_R + tid] = 0.f; }
+  const int Gd = a.G * a.dim, Gv = a.G * a.vdim;
+  const float* kb = a.k + ((int64_t)seq * a.t_max + t0) * Gd + (int64_t)g * a.dim;
+  const float* vb = a.v + ((int64_t)seq * a.t_max + t0) * Gv + (int64_t)g * a.vdim;
+  const float* pkb = a.pk ? a.pk + (int64_t)seq * a.n_pool_max * Gd + (int64_t)g * a.dim : nullptr;
+  const float* pvb = a.pv ? a.pv + (int64_t)seq * a.n_pool_max * Gv + (int64_t)g * a.vdim : nullptr;
+  const int n_out = R * a.vdim;
+  float acc[ATT_NOUT];
+#pragma unroll
+  for (int o = 0; o < ATT_NOUT; ++o) acc[o] = 0.f;
+  __syncthreads();
+  for (int j0 = 0; j0 < nk; j0 += ATT_TILE) {
+    const int nt = min(ATT_TILE, nk - j0);
+    // scores of this thread's key
+    if (tid < nt) {
+      const int j = j0 + tid;
+      const float* kp = j < nb ? pkb + (int64_t)j * Gd : kb + (int64_t)(j - nb) * Gd;
+      float s[ATT_R];
+#pragma unroll
+      for (int r = 0; r < ATT_R; ++r) s[r] = 0.f;
+      for (int d = 0; d < a.dim; ++d) {
+        const float kv = kp[d];
+#pragma unroll
+        for (int r = 0; r < ATT_R; ++r)
+          if (r < R) s[r] = fmaf(qs[r * a.dim + d], kv, s[r]);
+      }
+#pragma unroll
+      for (int r = 0; r < ATT_R; ++r)
+        if (r < R) sc[r * ATT_TILE + tid] = s[r];
+    }
+    __syncthreads();
+    // statistics: wave w owns heads w, w + 4
+    for (int r = tid >> 6; r < R; r += 4) {
+      const int lane = tid & 63;
+      float mx = -INFINITY;
+      for (int i = lane; i < nt; i += 64) mx = fmaxf(mx, sc[r * ATT_TILE + i]);
+      mx = wave_max(mx);
+      const float m_old = stat[r], m_new = fmaxf(m_old, mx);
+      float sum = 0.f;
+      for (int i = lane; i < nt; i += 64) {
+        const float p = expf(sc[r * ATT_TILE + i] - m_new);
+        sc[r * ATT_TILE + i] = p;
+        sum += p;
+      }
+      sum = wave_sum(sum);
+      if (lane == 0) {
+        const float alpha = expf(m_old - m_new);          // first tile: exp(-inf) = 0
+        stat[r] = m_new;
+        stat[ATT_R + r] = stat[ATT_R + r] * alpha + sum;
+        stat[2 * ATT_R + r] = alpha;
+      }
+    }
+    __syncthreads();
+    // weighted values: thread -> output columns o = tid + 256 i of [R][vdim]
+#pragma unroll
+    for (int o = 0; o < ATT_NOUT; ++o) {
+      const int e = tid + 256 * o;
+      if (e >= n_out) break;
+      const int r = e / a.vdim, c = e - r * a.vdim;
+      float t = acc[o] * stat[2 * ATT_R + r];
+      const float* pr = sc + r * ATT_TILE;
+      for (int i = 0; i < nt; ++i) {
+        const int j = j0 + i;
+        const float* vp = j < nb ? pvb + (int64_t)j * Gv : vb + (int64_t)(j - nb) * Gv;
+        t = fmaf(pr[i], vp[c], t);
+      }
+      acc[o] = t;
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int o = 0; o < ATT_NOUT; ++o) {
+    const int e = tid + 256 * o;
+    if (e >= n_out) break;
+    const int r = e / a.vdim;
+    const float val = acc[o] / stat[ATT_R + r] * a.out_scale;
+    const int64_t col = (int64_t)h0 * a.vdim + e;
+    if (a.out) a.out[(int64_t)m * a.ldo + col] = val;
+    if (a.out16) a.out16[(int64_t)m * a.ldo16 + col] = f32_to_bf16(val);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// minGRU: grid (ceil(n / 256), M); the workgroup of a sequence's FIRST row in the step walks that sequence's rows
+__global__ __launch_bounds__(256) void mingru_kernel(const float* __restrict__ zx, int64_t ldzx, const float* __restrict__ g, int64_t ldg,
+                                                     float* __restrict__ state, const int32_t* __restrict__ row_seq,
+                                                     const int32_t* __restrict__ row_slot, const int32_t* __restrict__ row_back,
+                                                     float out_scale, float* __restrict__ out, int64_t ldo, bf16_t* __restrict__ out16,
+                                                     int64_t ldo16, int M, int n) {
+  const int m0 = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (row_back[m0] != 0 || c >= n) return;
+  float* sp = state + (int64_t)row_seq[m0] * n + c;
+  float S = row_slot[m0] == 0 ? 0.f : *sp;
+  for (int m = m0; m < M && row_back[m] == m - m0; ++m) {
+    const float z = sigmoid_f(zx[(int64_t)m * ldzx + c]);
+    const float u = zx[(int64_t)m * ldzx + n + c];
+    const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+    S = (1.0f - z) * S + z * cand;
+    const float o = out_scale * S * silu_f(g[(int64_t)m * ldg + c]);
+    if (out) out[(int64_t)m * ldo + c] = o;
+    if (out16) out16[(int64_t)m * ldo16 + c] = f32_to_bf16(o);
+  }
+  *sp = S;
+}
+
+// one wave per row: `top` rounds of arg-max (ties: the lower index), then the softmax over the chosen logits.  Lane l owns the
+// logits l, l + 64, ... and a bit per owned logit that says it has been chosen (E <= 4096).
+__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int64_t ld, int M, int E, int top,
+                                                          int32_t* __restrict__ idx, float* __restrict__ w) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= M) return;
+  const float* z = logits + (int64_t)row * ld;
+  int32_t* ir = idx + (int64_t)row * top;
+  float* wr = w + (int64_t)row * top;
+  uint64_t taken = 0;
+  float first = 0.f, sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane, i = 0; e < E; e += 64, ++i) {
+      const float v = z[e];
+      if (!((taken >> i) & 1) && (v > best || (v == best && e < bi) || bi == 0x7fffffff)) { best = v; bi = e; }
+    }
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float ob = __shfl_xor(best, off);
+      const int oi = __shfl_xor(bi, off);
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) { best = ob; bi = oi; }
+    }
+    if ((bi & 63) == lane) taken |= (uint64_t)1 << (bi >> 6);
+    if (k == 0) first = best;
+    const float p = expf(best - first);
+    sum += p;
+    if (lane == 0) { ir[k] = bi; wr[k] = p; }
+  }
+  // lane 0 wrote the unnormalised weights and is the one that scales them
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) wr[k] = wr[k] / sum;
+}
+
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ x, int64_t ldx, float* __restrict__ y, int64_t ldy,
+                                                       bf16_t* __restrict__ y16, int64_t ldy16, int n) {
+  const int m = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= n) return;
+  const float o = silu_f(x[(int64_t)m * ldx + c]) * x[(int64_t)m * ldx + n + c];
+  if (y) y[(int64_t)m * ldy + c] = o;
+  if (y16) y16[(int64_t)m * ldy16 + c] = f32_to_bf16(o);
+}
+
+// one wave per output value: grid (ceil(N / 4), Z).  VEC: rows of K % 8 == 0 values at 16-byte aligned addresses, 8 weights per load
+template <bool VEC>
+__global__ __launch_bounds__(256) void gemv_indexed_kernel(const float* __restrict__ A, int64_t lda, int a_div, const bf16_t* __restrict__ W,
+                                                           int64_t ldw, int64_t w_bs, const int32_t* __restrict__ w_idx,
+                                                           float* __restrict__ C, int64_t ldc, int N, int K) {
+  const int z = blockIdx.y, n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (n >= N) return;
+  const float* ar = A + (int64_t)(z / a_div) * lda;
+  const bf16_t* wr = W + (int64_t)w_idx[z] * w_bs + (int64_t)n * ldw;
+  float acc = 0.f;
+  if (VEC) {
+    for (int k = lane * 8; k < K; k += 512) {
+      const uint4 wv = *reinterpret_cast<const uint4*>(wr + k);
+      const float4 a0 = *reinterpret_cast<const float4*>(ar + k), a1 = *reinterpret_cast<const float4*>(ar + k + 4);
+      acc = fmaf(a0.x, bf16lo_to_f32(wv.x), acc); acc = fmaf(a0.y, bf16hi_to_f32(wv.x), acc);
+      acc = fmaf(a0.z, bf16lo_to_f32(wv.y), acc); acc = fmaf(a0.w, bf16hi_to_f32(wv.y), acc);
+      acc = fmaf(a1.x, bf16lo_to_f32(wv.z), acc); acc = fmaf(a1.y, bf16hi_to_f32(wv.z), acc);
+      acc = fmaf(a1.z, bf16lo_to_f32(wv.w), acc); acc = fmaf(a1.w, bf16hi_to_f32(wv.w), acc);
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) acc = fmaf(ar[k], bf16_to_f32(wr[k]), acc);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) C[(int64_t)z * ldc + n] = acc;
+}
+
+__global__ __launch_bounds__(256) void moe_combine_residual_kernel(float* __restrict__ x, int64_t ldx, const float* __restrict__ y,
+                                                                   int64_t ldy, const int32_t* __restrict__ slot_of,
+                                                                   const float* __restrict__ w, int top, const float* __restrict__ shared,
+                                                                   int64_t lds, const float* __restrict__ sg, int64_t ldsg, float mult,
+                                                                   int n) {
+  const int m = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= n) return;
+  float acc = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const int z = m * top + j;
+    const int64_t r = slot_of ? slot_of[z] : z;
+    acc = fmaf(w[z], y[r * ldy + c], acc);
+  }
+  if (shared) acc += (sg ? sigmoid_f(sg[(int64_t)m * ldsg]) : 1.0f) * shared[(int64_t)m * lds + c];
+  x[(int64_t)m * ldx + c] += mult * acc;
+}
+
+}  // namespace
+
+extern "C" int mn_axpy_rms_rows(float* x, int64_t ldx, const float* y, int64_t ldy, float mult, const uint16_t* w, float eps, float* n_out,
+                                int64_t ldn, uint16_t* n16, int64_t ldn16, int M, int n, void* stream) {
+  MN_CHECK_ARG(x && M >= 1 && n >= 1 && (w || (!n_out && !n16)), "mn_axpy_rms_rows: bad args");
+  hipLaunchKernelGGL(axpy_rms_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), x, ldx, y, ldy, mult, w, eps, n_out,
+                     ldn, n16, ldn16, M, n);
+  MN_CHECK_LAUNCH("mn_axpy_rms_rows");
+  return MN_OK;
+}
+
+extern "C" int mn_axpy_rms_filter_rows(float* x, int64_t ldx, const float* y, int64_t ldy, float mult, const uint16_t* w, float eps,
+                                       const uint16_t* taps_w, int taps, float* state, const int32_t* row_seq, const int32_t* row_slot,
+                                       float* h, int64_t ldh, int M, int n, void* stream) {
+  MN_CHECK_ARG(x && w && h && M >= 1 && n >= 1 && n <= 8192, "mn_axpy_rms_filter_rows: bad args (n=%d: at most 8192)", n);
+  MN_CHECK_ARG(!taps_w || (taps >= 1 && taps <= FUSED_MAX_TAPS && row_seq && row_slot && (taps == 1 || state)),
+               "mn_axpy_rms_filter_rows: bad filter (taps=%d: at most %d)", taps, FUSED_MAX_TAPS);
+  AxpyRmsFilterArgs a{x, ldx, y, ldy, mult, w, eps, taps_w, taps_w ? taps : 0, state, row_seq, row_slot, h, ldh, n};
+  const int vpt = (n + 255) / 256;
+  hipStream_t st = mn_stream(stream);
+#define MN_RB(V_) hipLaunchKernelGGL((axpy_rms_filter_kernel<V_>), dim3((unsigned)M), dim3(256), 0, st, a)
+  if (vpt <= 1) MN_RB(1); else if (vpt <= 2) MN_RB(2); else if (vpt <= 4) MN_RB(4); else if (vpt <= 8) MN_RB(8);
+  else if (vpt <= 16) MN_RB(16); else MN_RB(32);
+#undef MN_RB
+  MN_CHECK_LAUNCH("mn_axpy_rms_filter_rows");
+  return MN_OK;
+}
+
+extern "C" int mn_rope_unit_append(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, int rot_dims, const float* freq,
+                                   float mag, int unit, float eps, float q_scale, const int32_t* row_seq, const int32_t* row_slot,
+                                   float* q_out, int64_t ldq, float* k_arena, float* v_arena, int t_max, void* stream) {
+  MN_CHECK_ARG(qkv && row_seq && row_slot && q_out && k_arena && v_arena && M >= 1 && M <= 65535 && H >= 1 && G >= 1 && t_max >= 1,
+               "mn_rope_unit_append: bad args");
+  MN_CHECK_ARG(dim >= 1 && dim <= 512 && vdim >= 1 && rot_dims >= 0 && rot_dims <= dim && (rot_dims % 2) == 0 && (rot_dims == 0 || freq),
+               "mn_rope_unit_append: dim=%d (at most 512), rot_dims=%d (even, at most dim)", dim, rot_dims);
+  RopeArgs a{qkv, ldqkv, H, G, dim, vdim, rot_dims, freq, mag, unit, eps, q_scale, row_seq, row_slot, q_out, ldq, k_arena, v_arena, t_max};
+  hipLaunchKernelGGL(rope_unit_append_kernel, dim3((unsigned)mn_cdiv(H + 2 * G, 4), (unsigned)M), dim3(256), 0, mn_stream(stream), a, M);
+  MN_CHECK_LAUNCH("mn_rope_unit_append");
+  return MN_OK;
+}
+
+extern "C" int mn_pool_blocks_update(const float* k_arena, const float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool,
+                                     int Gd, int Gv, const int32_t* row_seq, const int32_t* row_slot, int M, void* stream) {
+  MN_CHECK_ARG(k_arena && v_arena && pk && pv && row_seq && row_slot && pool >= 1 && n_pool_max >= 1 && Gd >= 1 && Gv >= 1 && M >= 1 &&
+                   M <= 65535, "mn_pool_blocks_update: bad args");
+  hipLaunchKernelGGL(pool_blocks_kernel, dim3((unsigned)mn_cdiv(Gd + Gv, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), k_arena,
+                     v_arena, t_max, pk, pv, n_pool_max, pool, Gd, Gv, row_seq, row_slot);
+  MN_CHECK_LAUNCH("mn_pool_blocks_update");
+  return MN_OK;
+}
+
+extern "C" int mn_window_pool_attn(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk, const float* pv,
+                                   const int32_t* row_seq, const int32_t* row_slot, int M, int H, int G, int dim, int vdim, int t_max,
+                                   int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                                   int64_t ldo16, void* stream) {
+  MN_CHECK_ARG(q && k_arena && v_arena && row_seq && row_slot && (out || out16) && M >= 1 && H >= 1 && G >= 1 && (H % G) == 0 && dim >= 1 &&
+                   vdim >= 1 && t_max >= 1 && window >= 0 && pool >= 0, "mn_window_pool_attn: bad args");
+  MN_CHECK_ARG(pool == 0 || (window > 0 && pk && pv && n_pool_max >= 1), "mn_window_pool_attn: pooled blocks need a window and their arenas");
+  const int rep = H / G, chunks = (rep + ATT_R - 1) / ATT_R;
+  MN_CHECK_ARG((rep < ATT_R ? rep : ATT_R) * vdim <= ATT_NOUT * 256, "mn_window_pool_attn: vdim=%d too large", vdim);
+  const size_t lds = ((size_t)ATT_R * dim + ATT_R * ATT_TILE + 3 * ATT_R) * sizeof(float);
+  MN_CHECK_ARG(lds <= 64 * 1024, "mn_window_pool_attn: dim=%d too large", dim);
+  AttnArgs a{q, ldq, k_arena, v_arena, pool ? pk : nullptr, pool ? pv : nullptr, row_seq, row_slot, H, G, dim, vdim, t_max, n_pool_max, window,
+             pool, out_scale, out, ldo, out16, ldo16};
+  hipLaunchKernelGGL(window_pool_attn_kernel, dim3((unsigned)M, (unsigned)(G * chunks)), dim3(256), lds, mn_stream(stream), a);
+  MN_CHECK_LAUNCH("mn_window_pool_attn");
+  return MN_OK;
+}
+
+extern "C" int mn_mingru_rows(const float* zx, int64_t ldzx, const float* g, int64_t ldg, float* state, const int32_t* row_seq,
+                              const int32_t* row_slot, const int32_t* row_back, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                              int64_t ldo16, int M, int n, void* stream) {
+  MN_CHECK_ARG(zx && g && state && row_seq && row_slot && row_back && (out || out16) && M >= 1 && M <= 65535 && n >= 1,
+               "mn_mingru_rows: bad args");
+  hipLaunchKernelGGL(mingru_kernel, dim3((unsigned)mn_cdiv(n, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), zx, ldzx, g, ldg, state,
+                     row_seq, row_slot, row_back, out_scale, out, ldo, out16, ldo16, M, n);
+  MN_CHECK_LAUNCH("mn_mingru_rows");
+  return MN_OK;
+}
+
+extern "C" int mn_router_topk_rows(const float* logits, int64_t ld, int M, int E, int top, int32_t* idx, float* w, void* stream) {
+  MN_CHECK_ARG(logits && idx && w && M >= 1 && E >= 1 && E <= 4096 && top >= 1 && top <= E, "mn_router_topk_rows: bad args (E=%d top=%d)", E, top);
+  hipLaunchKernelGGL(router_topk_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), logits, ld, M, E, top, idx, w);
+  MN_CHECK_LAUNCH("mn_router_topk_rows");
+  return MN_OK;
+}
+
+extern "C" int mn_silu_mul_rows(const float* x, int64_t ldx, float* y, int64_t ldy, uint16_t* y16, int64_t ldy16, int M, int n,
+                                void* stream) {
+  MN_CHECK_ARG(x && (y || y16) && M >= 1 && M <= 65535 && n >= 1, "mn_silu_mul_rows: bad args");
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)mn_cdiv(n, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), x, ldx, y, ldy, y16,
+                     ldy16, n);
+  MN_CHECK_LAUNCH("mn_silu_mul_rows");
+  return MN_OK;
+}
+
+extern "C" int mn_gemv_f32_indexed(const float* A, int64_t lda, int a_div, const uint16_t* W, int64_t ldw, int64_t w_bs,
+                                   const int32_t* w_idx, float* C, int64_t ldc, int Z, int N, int K, void* stream) {
+  MN_CHECK_ARG(A && W && w_idx && C && a_div >= 1 && Z >= 1 && Z <= 65535 && N >= 1 && K >= 1, "mn_gemv_f32_indexed: bad args (Z=%d)", Z);
+  const bool vec = (K % 8) == 0 && (ldw % 8) == 0 && (w_bs % 8) == 0 && (lda % 4) == 0 && (((uintptr_t)W | (uintptr_t)A) & 15) == 0;
+  const dim3 grid((unsigned)mn_cdiv(N, 4), (unsigned)Z);
+  if (vec) hipLaunchKernelGGL((gemv_indexed_kernel<true>), grid, dim3(256), 0, mn_stream(stream), A, lda, a_div, W, ldw, w_bs, w_idx, C, ldc, N, K);
+  else hipLaunchKernelGGL((gemv_indexed_kernel<false>), grid, dim3(256), 0, mn_stream(stream), A, lda, a_div, W, ldw, w_bs, w_idx, C, ldc, N, K);
+  MN_CHECK_LAUNCH("mn_gemv_f32_indexed");
+  return MN_OK;
+}
+
+extern "C" int mn_moe_combine_residual(float* x, int64_t ldx, const float* y, int64_t ldy, const int32_t* slot_of, const float* w, int top,
+                                       const float* shared, int64_t lds, const float* sg, int64_t ldsg, float mult, int M, int n,
+                                       void* stream) {
+  MN_CHECK_ARG(x && y && w && top >= 1 && M >= 1 && M <= 65535 && n >= 1, "mn_moe_combine_residual: bad args");
+  hipLaunchKernelGGL(moe_combine_residual_kernel, dim3((unsigned)mn_cdiv(n, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), x, ldx, y,
+                     ldy, slot_of, w, top, shared, lds, sg, ldsg, mult, n);
+  MN_CHECK_LAUNCH("mn_moe_combine_residual");
+  return MN_OK;
+}

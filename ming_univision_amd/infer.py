@@ -43,13 +43,17 @@ def load_safetensors_dir(path):
 
 def load_model(path, dtype="bf16", device="cuda", **kw):
     """The served model of a checkpoint directory, its class chosen by config.json (configuration.MODEL_REGISTRY):
-    "pizitar" -> PizitarForCausalLM (dtype "bf16" | "f32" = its matrix-product arithmetic; kw: t_max, eos_token_id),
+    "pizitar" -> PizitarForCausalLM, "sakinex" -> SakinexForCausalLM (dtype "bf16" | "f32" = the matrix-product arithmetic; kw: t_max,
+    eos_token_id),
     "ming_univision" -> MingUniVisionInfer (dtype = the weight format)."""
     from .configuration import config_from_pretrained
     name, _ = config_from_pretrained(path)
     if name == "pizitar":
         from .pizitar import PizitarForCausalLM
         return PizitarForCausalLM.from_pretrained(path, device=device, arith=dtype, **kw)
+    if name == "sakinex":
+        from .sakinex import SakinexForCausalLM
+        return SakinexForCausalLM.from_pretrained(path, device=device, arith=dtype, **kw)
     return MingUniVisionInfer(path, dtype=dtype, device=device, **kw)
 
 
