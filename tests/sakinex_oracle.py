@@ -94,15 +94,15 @@ def visible(i, mask):
     return toks, blocks
 
 
-def windowed_attention(q, k, v, scale, mask):
+def windowed_attention(q, k, v, scale, mask, rows=None):
     """q [T, H, d], k [T, G, d], v [T, G, e] as the cache holds them -> [T, H, e].  Tokens in the window and the means of the
-    whole blocks before it share one softmax."""
+    whole blocks before it share one softmax.  rows: the positions to evaluate (default all; the others stay zero)."""
     T, H, _ = q.shape
     G = k.shape[1]
     rep = H // G
     P = int(mask["pool"]) if mask and mask.get("pool") else 0
     out = torch.zeros(T, H, v.shape[2], dtype=q.dtype)
-    for i in range(T):
+    for i in (range(T) if rows is None else rows):
         toks, blocks = visible(i, mask)
         for h in range(H):
             g = h // rep
