@@ -914,12 +914,32 @@ MN_API int mn_window_pool_attn(const float* q, int64_t ldq, const float* k_arena
                                const int32_t* row_seq, const int32_t* row_slot, int M, int H, int G, int dim, int vdim, int t_max,
                                int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo, uint16_t* out16,
                                int64_t ldo16, void* stream);
+/* The same attention in its tiled form (what mn_pmix_step runs; mn_window_pool_attn is the plain kernel it is checked against): a
+ * workgroup takes a run of up to mn_window_attn_block_rows() consecutive rows of ONE sequence at consecutive positions (blk_tab int32
+ * [n_blk, 2] = (first row, rows)), or single rows (one_row = 1: row b is block b, blk_tab unused), and shares each 64-key tile of the
+ * run among its rows and query heads.  nsplit > 1 cuts a run's keys over nsplit workgroups and merges their partial softmaxes in a
+ * second launch (mn_window_attn_splits proposes it from the launch size and max_keys, the most keys any run sees; workspace from
+ * mn_window_attn_workspace_bytes).  vdim <= 512. */
+MN_API int mn_window_attn_block_rows(void);
+MN_API int mn_window_attn_splits(int n_blk, int H, int G, int one_row, int max_keys);
+MN_API size_t mn_window_attn_workspace_bytes(int n_blk, int H, int G, int vdim, int one_row, int nsplit);
+MN_API int mn_window_pool_attn_blocks(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk,
+                                      const float* pv, const int32_t* row_seq, const int32_t* row_slot, const int32_t* blk_tab, int n_blk,
+                                      int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
+                                      float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
+                                      size_t workspace_bytes, void* stream);
 /* minGRU over each sequence's rows: z = sigmoid(zx[m, c]), u = zx[m, n + c] (biases already added), candidate = u + 1/2 (u >= 0) or
  * sigmoid(u); S = (1 - z) S + z candidate from state fp32 [n_seq, n] (a row at slot 0 starts from zero), which is left at the
  * sequence's last row; out[m, c] = out_scale * S * silu(g[m, c]).  Rows of one sequence are consecutive (row_back as in 9). */
 MN_API int mn_mingru_rows(const float* zx, int64_t ldzx, const float* g, int64_t ldg, float* state, const int32_t* row_seq,
                           const int32_t* row_slot, const int32_t* row_back, float out_scale, float* out, int64_t ldo, uint16_t* out16,
                           int64_t ldo16, int M, int n, void* stream);
+/* The same as a chunked scan (three launches: per-chunk products and sums, a carry over the chunks, the outputs): the form for steps
+ * of many rows, where one thread walking all rows of a sequence is a chain of M dependent steps.  out (fp32) is required. */
+MN_API size_t mn_mingru_scan_workspace_bytes(int M, int n);
+MN_API int mn_mingru_rows_scan(const float* zx, int64_t ldzx, const float* g, int64_t ldg, float* state, const int32_t* row_seq,
+                               const int32_t* row_slot, const int32_t* row_back, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                               int64_t ldo16, int M, int n, void* workspace, size_t workspace_bytes, void* stream);
 /* The `top` largest of logits[m, 0 .. E) (ties: the lower index) and the softmax over those alone: idx int32 [M, top], w fp32 [M, top] */
 MN_API int mn_router_topk_rows(const float* logits, int64_t ld, int M, int E, int top, int32_t* idx, float* w, void* stream);
 /* y[m, c] = silu(x[m, c]) * x[m, n + c]; y16: optional bf16 copy */
@@ -975,11 +995,14 @@ MN_API size_t mn_sizeof_pmix_layer(void);
 MN_API size_t mn_sizeof_pmix_model(void);
 MN_API size_t mn_sizeof_pmix_state(void);
 /* One pass of the stack over M rows; rows, row arrays, out and trace as mn_seq_step (trace: fp32 [n_runs, M, width]).
- * flags: MN_SEQ_ROWS_DISTINCT fuses the residual add / norm / filter launches of decode rows. */
+ * blk_tab / n_blk: the rows cut into runs of <= mn_window_attn_block_rows() consecutive rows of one sequence (unused with
+ * MN_SEQ_ROWS_DISTINCT); max_len >= every position + 1 (it sizes the attention's key splits).
+ * flags: MN_SEQ_ROWS_DISTINCT = every row is alone in its sequence (a decode step): the residual add / norm / filter launches are
+ * fused and the attention takes the rows one by one. */
 MN_API size_t mn_pmix_workspace_bytes(const mn_pmix_model* m, int M);
 MN_API int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
-                        const int32_t* row_slot, const int32_t* row_back, int flags, float* out, float* trace, void* workspace,
-                        size_t workspace_bytes, void* stream);
+                        const int32_t* row_slot, const int32_t* row_back, const int32_t* blk_tab, int n_blk, int max_len, int flags,
+                        float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

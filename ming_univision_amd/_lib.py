@@ -317,12 +317,19 @@ SYMBOLS = {
     "mn_pool_blocks_update": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p]),
     "mn_window_pool_attn": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64, _p]),
     "mn_mingru_rows": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _f, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_mingru_scan_workspace_bytes": (_sz, [_i, _i]),
+    "mn_mingru_rows_scan": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _f, _p, _i64, _p, _i64, _i, _i, _p, _sz, _p]),
     "mn_router_topk_rows": (_i, [_p, _i64, _i, _i, _i, _p, _p, _p]),
     "mn_silu_mul_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _i, _i, _p]),
     "mn_gemv_f32_indexed": (_i, [_p, _i64, _i, _p, _i64, _i64, _p, _p, _i64, _i, _i, _i, _p]),
     "mn_moe_combine_residual": (_i, [_p, _i64, _p, _i64, _p, _p, _i, _p, _i64, _p, _i64, _f, _i, _i, _p]),
     "mn_pmix_workspace_bytes": (_sz, [C.POINTER(PmixModel), _i]),
-    "mn_pmix_step": (_i, [C.POINTER(PmixModel), C.POINTER(PmixState), _p, _i64, _i, _p, _p, _p, _i, _p, _p, _p, _sz, _p]),
+    "mn_pmix_step": (_i, [C.POINTER(PmixModel), C.POINTER(PmixState), _p, _i64, _i, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
+    "mn_window_attn_block_rows": (_i, []),
+    "mn_window_attn_splits": (_i, [_i, _i, _i, _i, _i]),
+    "mn_window_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "mn_window_pool_attn_blocks": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64, _i,
+                                        _p, _sz, _p]),
     "mn_semdec_step": (_i, [C.POINTER(SemDec), _p, _i, _p, _p, _p, _p, _i, _i64, _p, _p, _p, _sz, _p]),
 }
 

@@ -27,7 +27,7 @@ PDims pdims(const mn_pmix_layer& l) {
 
 struct PPlan {
   int n_in = 1, cqkv = 1, cq = 1, n_cat = 1, n_ff_in = 1, sff = 1, top = 1, ff = 1, experts = 1;
-  size_t gemm_ws = 0;
+  size_t gemm_ws = 0, attn_ws = 0, gru_ws = 0;
 };
 
 bool grouped_route(const mn_pmix_model* m, const mn_pmix_layer& l, int M) {
@@ -49,6 +49,11 @@ PPlan make_plan(const mn_pmix_model* m, int M) {
     if (l.top > p.top) p.top = l.top;
     if (l.ff > p.ff) p.ff = l.ff;
     if (l.experts > p.experts) p.experts = l.experts;
+    // key splits are chosen so that a launch has about two workgroups per compute unit: (runs x heads x splits) stays below four
+    const size_t aw = (size_t)4 * mn_num_cus() * 16 * (2 + (size_t)l.vdim) * sizeof(float);
+    if (aw > p.attn_ws) p.attn_ws = aw;
+    const size_t gw = mn_mingru_scan_workspace_bytes(M, l.gru);
+    if (gw > p.gru_ws) p.gru_ws = gw;
     if (m->arith == MN_SEQ_ARITH_BF16 && M > 8 && M <= 64) {       // scratch of the weight-streaming MFMA route: the largest product of the stack
       const int W = m->width;
       const int shapes[4][2] = {{d.n_in, W}, {W, d.n_cat}, {d.n_ff_in, W}, {W, l.shared_ff}};
@@ -86,19 +91,23 @@ extern "C" size_t mn_pmix_workspace_bytes(const mn_pmix_model* m, int M) {
   n += al(Z * W * 4);                                  // their results
   n += al(Z * W * 2);                                  // gathered bf16 rows
   n += 2 * al(((size_t)p.experts + 1) * 4) + 2 * al(Z * 4);   // counts, offsets, perm, slot_of
-  n += al(p.gemm_ws);
+  n += al(p.gemm_ws) + al(p.attn_ws) + al(p.gru_ws);
   return n;
 }
 
 extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
-                            const int32_t* row_slot, const int32_t* row_back, int flags, float* out, float* trace, void* workspace,
-                            size_t workspace_bytes, void* stream) {
+                            const int32_t* row_slot, const int32_t* row_back, const int32_t* blk_tab, int n_blk, int max_len, int flags,
+                            float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream) {
   MN_CHECK_ARG(m && st && m->layers && m->run_layer && m->run_readd && m->final_w && x && row_seq && row_slot && row_back && out && workspace,
                "mn_pmix_step: null pointer");
   MN_CHECK_ARG(st->k && st->v && st->pk && st->pv && st->canon && st->conv && st->gru, "mn_pmix_step: null state table");
   MN_CHECK_ARG(M >= 1 && M <= 65535 && m->width >= 1 && m->n_layers >= 1 && m->n_runs >= 1 && m->taps >= 0,
                "mn_pmix_step: bad sizes (M=%d)", M);
   MN_CHECK_ARG(workspace_bytes >= mn_pmix_workspace_bytes(m, M), "mn_pmix_step: workspace too small");
+  const bool one_row = (flags & MN_SEQ_ROWS_DISTINCT) != 0;
+  MN_CHECK_ARG(one_row || (blk_tab && n_blk >= 1 && n_blk <= M), "mn_pmix_step: rows that share sequences need the table of their runs");
+  MN_CHECK_ARG(max_len >= 1 && max_len <= st->t_max, "mn_pmix_step: max_len=%d outside the cache (t_max=%d)", max_len, st->t_max);
+  if (one_row) n_blk = M;
   const PPlan p = make_plan(m, M);
   const int W = m->width, arith = m->arith;
   const size_t R = (size_t)M, Zmax = R * p.top;
@@ -133,6 +142,8 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
   int32_t* slot_of = (int32_t*)take(Zmax * 4);
   void* gws = p.gemm_ws ? take(p.gemm_ws) : nullptr;
   const size_t gwb = p.gemm_ws;
+  void* aws = take(p.attn_ws);
+  void* gruws = take(p.gru_ws);
   if (!want16) hh = cath = sah = nullptr;
   hipStream_t hs = mn_stream(stream);
   int rc;
@@ -202,11 +213,26 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
     if (l.pool > 0)
       MN_TRY(mn_pool_blocks_update(st->k[ri], st->v[ri], st->t_max, st->pk[ri], st->pv[ri], st->n_pool_max, l.pool, d.ck, d.cv, row_seq,
                                    row_slot, M, stream));
-    MN_TRY(mn_window_pool_attn(qf, d.cq, st->k[ri], st->v[ri], st->pk[ri], st->pv[ri], row_seq, row_slot, M, l.heads, l.kv_heads, l.dim,
-                               l.vdim, st->t_max, st->n_pool_max, l.window, l.pool, l.left_scale, cat, d.n_cat, cath, d.n_cat, stream));
+    {
+      const int rb = one_row ? 1 : mn_window_attn_block_rows();
+      int max_keys = max_len;
+      if (l.window > 0) {
+        max_keys = l.window + rb - 1 < max_len ? l.window + rb - 1 : max_len;
+        if (l.pool > 0) max_keys += max_len / l.pool;
+      }
+      int ns = mn_window_attn_splits(n_blk, l.heads, l.kv_heads, one_row, max_keys);
+      while (ns > 1 && mn_window_attn_workspace_bytes(n_blk, l.heads, l.kv_heads, l.vdim, one_row, ns) > p.attn_ws) --ns;
+      MN_TRY(mn_window_pool_attn_blocks(qf, d.cq, st->k[ri], st->v[ri], st->pk[ri], st->pv[ri], row_seq, row_slot, blk_tab, n_blk, one_row,
+                                        l.heads, l.kv_heads, l.dim, l.vdim, st->t_max, st->n_pool_max, l.window, l.pool, l.left_scale, cat,
+                                        d.n_cat, cath, d.n_cat, ns, aws, p.attn_ws, stream));
+    }
     const int hv = l.heads * l.vdim;
-    MN_TRY(mn_mingru_rows(pin + d.cqkv, d.n_in, pin + d.cqkv + 2 * l.gru, d.n_in, st->gru[ri], row_seq, row_slot, row_back, l.right_scale,
-                          cat + hv, d.n_cat, cath ? cath + hv : nullptr, d.n_cat, M, l.gru, stream));
+    if (M >= 2 * 32 && !one_row)                     // many rows: the recurrence as a chunked scan instead of one thread per channel walking them all
+      MN_TRY(mn_mingru_rows_scan(pin + d.cqkv, d.n_in, pin + d.cqkv + 2 * l.gru, d.n_in, st->gru[ri], row_seq, row_slot, row_back, l.right_scale,
+                                 cat + hv, d.n_cat, cath ? cath + hv : nullptr, d.n_cat, M, l.gru, gruws, p.gru_ws, stream));
+    else
+      MN_TRY(mn_mingru_rows(pin + d.cqkv, d.n_in, pin + d.cqkv + 2 * l.gru, d.n_in, st->gru[ri], row_seq, row_slot, row_back, l.right_scale,
+                            cat + hv, d.n_cat, cath ? cath + hv : nullptr, d.n_cat, M, l.gru, stream));
     MN_TRY(linear(arith, M, cat, d.n_cat, cath, d.n_cat, l.w_out, W, d.n_cat, nullptr, yf, W, gws, gwb, stream));
     pend = yf;
     // ---- feed-forward sublayer ----

@@ -8,7 +8,8 @@
 //   mn_rope_unit_append        rotary (frequency table) + unit-RMS per head on q and k, q scaled, k / v appended to their arenas
 //   mn_pool_blocks_update      mean key / value of the blocks a step completes
 //   mn_window_pool_attn        softmax over the window's tokens and the block means before it, online softmax in fp32
-//   mn_mingru_rows             S = (1 - z) S + z c over each sequence's rows, gated output
+//   mn_window_pool_attn_blocks the same, tiled: runs of rows and query heads share key tiles, key splits with a merge launch
+//   mn_mingru_rows             S = (1 - z) S + z c over each sequence's rows, gated output (mn_mingru_rows_scan: as a chunked scan)
 //   mn_router_topk_rows        top-k of the router logits, softmax over the chosen
 //   mn_silu_mul_rows           silu(gate) * up
 //   mn_gemv_f32_indexed        one row against the weight block an index names (experts of few rows, and the fp32 path)
@@ -328,6 +329,213 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(AttnArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
+// Attention, tiled form: one workgroup per (run of <= RB consecutive rows of one sequence, key/value head, chunk of query heads,
+// key split) holds AQ query vectors (rows x heads) in LDS and walks its share of the run's keys in tiles of 64 (block means first,
+// then the tokens from the first row's window start to the last row's position; what a row may not see is masked per (row, key)).
+// Scores: four threads per key, each a quarter of the head's values, all AQ vectors against the key in registers.  The tile's
+// softmax statistics are merged into the running ones by one wave per vector.  Values: a thread owns one output column (and a
+// share of the tile's keys when the head has fewer than 256 columns) for all AQ vectors.  With key splits the unnormalised sums
+// and statistics go to a workspace and a second launch merges them.
+constexpr int AKT = 64;
+struct AttnTArgs {
+  const float* q; int64_t ldq;
+  const float *k, *v, *pk, *pv;
+  const int32_t *row_seq, *row_slot, *blk_tab;
+  int H, G, dim, vdim, t_max, n_pool_max, window, pool, rows_per_blk, hpc, nsplit;
+  float out_scale;
+  float* out; int64_t ldo; bf16_t* out16; int64_t ldo16;
+  float* part;
+};
+
+__device__ __forceinline__ int win_t0(int pos, int window) { return window > 0 ? max(0, pos - window + 1) : 0; }
+__device__ __forceinline__ int win_nb(int pos, int window, int pool) {
+  return (window > 0 && pool > 0 && pos - window + 1 >= 0) ? (pos - window + 1) / pool : 0;
+}
+
+template <int AQ, bool VEC>
+__global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, b = blockIdx.x, gy = blockIdx.y, sp = blockIdx.z;
+  const int rep = a.H / a.G, chunks = (rep + a.hpc - 1) / a.hpc;
+  const int g = gy / chunks, h0 = g * rep + (gy % chunks) * a.hpc;
+  const int Rc = min(a.hpc, g * rep + rep - h0);
+  const int r0 = a.blk_tab ? a.blk_tab[2 * b] : b;
+  const int nr = a.blk_tab ? min(a.blk_tab[2 * b + 1], a.rows_per_blk) : 1;
+  const int nqv = nr * Rc;
+  const int seq = a.row_seq[r0], pos0 = a.row_slot[r0], posL = pos0 + nr - 1;
+  const int nbL = win_nb(posL, a.window, a.pool), tF = win_t0(pos0, a.window);
+  const int nk = nbL + (posL - tF + 1);
+  const int ntile = (nk + AKT - 1) / AKT, tps = (ntile + a.nsplit - 1) / a.nsplit;
+  const int tile0 = sp * tps, tile1 = min(ntile, tile0 + tps);
+  float* qs = lds;                          // [AQ][dim]
+  float* sc = qs + AQ * a.dim;              // [AQ][AKT]
+  float* pT = sc + AQ * AKT;                // [AKT][AQ]
+  float* st_m = pT + AKT * AQ;              // [AQ] running max, [AQ] running sum, [AQ] rescale of this tile
+  float* st_l = st_m + AQ;
+  float* st_a = st_l + AQ;
+  float* red = st_a + AQ;                   // [256 / cw][AQ][cw]
+  for (int e = tid; e < AQ * a.dim; e += 256) {
+    const int qv = e / a.dim, d = e - qv * a.dim;
+    qs[e] = qv < nqv ? a.q[(int64_t)(r0 + qv / Rc) * a.ldq + (int64_t)(h0 + qv % Rc) * a.dim + d] : 0.f;
+  }
+  if (tid < AQ) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_a[tid] = 0.f; }
+  const int Gd = a.G * a.dim, Gv = a.G * a.vdim;
+  const float* kb = a.k + ((int64_t)seq * a.t_max + tF) * Gd + (int64_t)g * a.dim;
+  const float* vb = a.v + ((int64_t)seq * a.t_max + tF) * Gv + (int64_t)g * a.vdim;
+  const float* pkb = a.pk ? a.pk + (int64_t)seq * a.n_pool_max * Gd + (int64_t)g * a.dim : nullptr;
+  const float* pvb = a.pv ? a.pv + (int64_t)seq * a.n_pool_max * Gv + (int64_t)g * a.vdim : nullptr;
+  constexpr int NCB = 2;                    // column blocks of 256: vdim <= 512
+  float acc[NCB][AQ];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+    for (int i = 0; i < AQ; ++i) acc[cb][i] = 0.f;
+  __syncthreads();
+  for (int tile = tile0; tile < tile1; ++tile) {
+    const int j0 = tile * AKT, nt = min(AKT, nk - j0);
+    {  // ---- scores ----
+      const int key = tid >> 2, part = tid & 3, j = j0 + key;
+      const bool valid = key < nt;
+      const float* kp = !valid ? kb : (j < nbL ? pkb + (int64_t)j * Gd : kb + (int64_t)(j - nbL) * Gd);
+      float s[AQ];
+#pragma unroll
+      for (int i = 0; i < AQ; ++i) s[i] = 0.f;
+      if (valid) {
+        if (VEC) {
+          for (int f = part; f < a.dim / 4; f += 4) {
+            const float4 kv = *reinterpret_cast<const float4*>(kp + 4 * f);
+#pragma unroll
+            for (int i = 0; i < AQ; ++i) {
+              const float4 qq = *reinterpret_cast<const float4*>(qs + i * a.dim + 4 * f);
+              s[i] = fmaf(qq.x, kv.x, s[i]); s[i] = fmaf(qq.y, kv.y, s[i]); s[i] = fmaf(qq.z, kv.z, s[i]); s[i] = fmaf(qq.w, kv.w, s[i]);
+            }
+          }
+        } else {
+          for (int d = part; d < a.dim; d += 4) {
+            const float kv = kp[d];
+#pragma unroll
+            for (int i = 0; i < AQ; ++i) s[i] = fmaf(qs[i * a.dim + d], kv, s[i]);
+          }
+        }
+      }
+      const int t = tF + (j - nbL);          // the token a non-pooled key index stands for
+#pragma unroll
+      for (int i = 0; i < AQ; ++i) {
+        float v = s[i];
+        v += __shfl_xor(v, 1);
+        v += __shfl_xor(v, 2);
+        if ((i & 3) == part) {
+          const int pos = pos0 + i / Rc;
+          const bool see = valid && i < nqv && (j < nbL ? j < win_nb(pos, a.window, a.pool) : (t >= win_t0(pos, a.window) && t <= pos));
+          sc[i * AKT + key] = see ? v : -INFINITY;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- statistics: wave w owns the vectors w, w + 4, ... ----
+    for (int i = tid >> 6; i < AQ; i += 4) {
+      const int lane = tid & 63;
+      const float x = sc[i * AKT + lane];
+      const float m_old = st_m[i], m_new = fmaxf(m_old, wave_max(x));
+      const float p = m_new == -INFINITY ? 0.f : expf(x - m_new);
+      const float sum = wave_sum(p);
+      pT[lane * AQ + i] = p;
+      if (lane == 0) {
+        const float alpha = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+        st_m[i] = m_new;
+        st_l[i] = st_l[i] * alpha + sum;
+        st_a[i] = alpha;
+      }
+    }
+    __syncthreads();
+    // ---- weighted values ----
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      const int c0 = cb * 256;
+      if (c0 >= a.vdim) break;
+      const int cw = min(256, a.vdim - c0), nsub = 256 / cw, c = tid % cw, ksub = tid / cw;
+      if (ksub < nsub) {
+#pragma unroll
+        for (int i = 0; i < AQ; ++i) acc[cb][i] *= st_a[i];
+        for (int jj = ksub; jj < nt; jj += nsub) {
+          const int j = j0 + jj;
+          const float vv = (j < nbL ? pvb + (int64_t)j * Gv : vb + (int64_t)(j - nbL) * Gv)[c0 + c];
+          const float* pr = pT + jj * AQ;
+#pragma unroll
+          for (int i = 0; i < AQ; i += 4) {
+            const float4 pp = *reinterpret_cast<const float4*>(pr + i);
+            acc[cb][i] = fmaf(pp.x, vv, acc[cb][i]); acc[cb][i + 1] = fmaf(pp.y, vv, acc[cb][i + 1]);
+            acc[cb][i + 2] = fmaf(pp.z, vv, acc[cb][i + 2]); acc[cb][i + 3] = fmaf(pp.w, vv, acc[cb][i + 3]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // ---- the key shares of a column meet in LDS; then the result, or this split's part of it ----
+  float* part_out = a.nsplit > 1 ? a.part + (((int64_t)b * gridDim.y + gy) * a.nsplit + sp) * ((int64_t)AQ * (2 + a.vdim)) : nullptr;
+  if (part_out && tid < AQ) { part_out[tid] = st_m[tid]; part_out[AQ + tid] = st_l[tid]; }
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int c0 = cb * 256;
+    if (c0 >= a.vdim) break;
+    const int cw = min(256, a.vdim - c0), nsub = 256 / cw, c = tid % cw, ksub = tid / cw;
+    if (ksub < nsub) {
+#pragma unroll
+      for (int i = 0; i < AQ; ++i) red[(ksub * AQ + i) * cw + c] = acc[cb][i];
+    }
+    __syncthreads();
+    for (int e = tid; e < nqv * cw; e += 256) {
+      const int i = e / cw, cc = e - i * cw;
+      float t = 0.f;
+      for (int u = 0; u < nsub; ++u) t += red[(u * AQ + i) * cw + cc];
+      if (part_out) {
+        part_out[2 * AQ + (int64_t)i * a.vdim + c0 + cc] = t;
+      } else {
+        const float val = t / st_l[i] * a.out_scale;
+        const int64_t col = (int64_t)(h0 + i % Rc) * a.vdim + c0 + cc;
+        const int row = r0 + i / Rc;
+        if (a.out) a.out[(int64_t)row * a.ldo + col] = val;
+        if (a.out16) a.out16[(int64_t)row * a.ldo16 + col] = f32_to_bf16(val);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// grid (n_blk, G * chunks): the splits' statistics and sums of every vector become its result
+template <int AQ>
+__global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
+  const int tid = threadIdx.x, b = blockIdx.x, gy = blockIdx.y;
+  const int rep = a.H / a.G, chunks = (rep + a.hpc - 1) / a.hpc;
+  const int g = gy / chunks, h0 = g * rep + (gy % chunks) * a.hpc;
+  const int Rc = min(a.hpc, g * rep + rep - h0);
+  const int r0 = a.blk_tab ? a.blk_tab[2 * b] : b;
+  const int nr = a.blk_tab ? min(a.blk_tab[2 * b + 1], a.rows_per_blk) : 1;
+  const int nqv = nr * Rc;
+  const int64_t stride = (int64_t)AQ * (2 + a.vdim);
+  const float* base = a.part + ((int64_t)b * gridDim.y + gy) * a.nsplit * stride;
+  for (int e = tid; e < nqv * a.vdim; e += 256) {
+    const int i = e / a.vdim, c = e - i * a.vdim;
+    float mx = -INFINITY;
+    for (int s = 0; s < a.nsplit; ++s) mx = fmaxf(mx, base[s * stride + i]);
+    float L = 0.f, t = 0.f;
+    for (int s = 0; s < a.nsplit; ++s) {
+      const float ms = base[s * stride + i];
+      if (ms == -INFINITY) continue;
+      const float w = expf(ms - mx);
+      L = fmaf(base[s * stride + AQ + i], w, L);
+      t = fmaf(base[s * stride + 2 * AQ + (int64_t)i * a.vdim + c], w, t);
+    }
+    const float val = t / L * a.out_scale;
+    const int64_t col = (int64_t)(h0 + i % Rc) * a.vdim + c;
+    const int row = r0 + i / Rc;
+    if (a.out) a.out[(int64_t)row * a.ldo + col] = val;
+    if (a.out16) a.out16[(int64_t)row * a.ldo16 + col] = f32_to_bf16(val);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
 // minGRU: grid (ceil(n / 256), M); the workgroup of a sequence's FIRST row in the step walks that sequence's rows
 __global__ __launch_bounds__(256) void mingru_kernel(const float* __restrict__ zx, int64_t ldzx, const float* __restrict__ g, int64_t ldg,
                                                      float* __restrict__ state, const int32_t* __restrict__ row_seq,
@@ -348,6 +556,79 @@ __global__ __launch_bounds__(256) void mingru_kernel(const float* __restrict__ z
     if (out16) out16[(int64_t)m * ldo16 + c] = f32_to_bf16(o);
   }
   *sp = S;
+}
+
+// minGRU as a chunked scan, for steps of many rows.  Over ALL rows of the step the recurrence is S_m = a_m S_(m-1) + b_m with
+// a = 1 - z, b = z * candidate, where a sequence's first row in the step takes a = 0 and b = (1 - z) S_start + z * candidate
+// (S_start: the sequence's stored state, zero at position 0).  Pass 1: every chunk of MG_CH rows -> (product of a, scan from zero),
+// and S_start of the first rows parked in their output rows.  Pass 2: one thread per channel carries S over the chunks.  Pass 3:
+// every chunk again from its carried S, writing the outputs and, at a sequence's last row, its state.
+constexpr int MG_CH = 32;
+struct MinGruArgs {
+  const float* zx; int64_t ldzx;
+  const float* g; int64_t ldg;
+  float* state; const int32_t *row_seq, *row_slot, *row_back;
+  float out_scale;
+  float* out; int64_t ldo; bf16_t* out16; int64_t ldo16;
+  float* ws;            // [n_chunks][2][n]
+  int M, n;
+};
+
+__device__ __forceinline__ void mingru_ab(const MinGruArgs& a, int m, int c, float s_start, float& av, float& bv) {
+  const float z = sigmoid_f(a.zx[(int64_t)m * a.ldzx + c]);
+  const float u = a.zx[(int64_t)m * a.ldzx + a.n + c];
+  const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+  av = 1.0f - z;
+  bv = z * cand;
+  if (a.row_back[m] == 0) { bv = av * s_start + bv; av = 0.f; }
+}
+
+__global__ __launch_bounds__(256) void mingru_pass1_kernel(MinGruArgs a) {
+  const int ch = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= a.n) return;
+  const int m0 = ch * MG_CH, m1 = min(a.M, m0 + MG_CH);
+  float A = 1.f, B = 0.f;
+  for (int m = m0; m < m1; ++m) {
+    float s_start = 0.f;
+    if (a.row_back[m] == 0) {
+      s_start = a.row_slot[m] == 0 ? 0.f : a.state[(int64_t)a.row_seq[m] * a.n + c];
+      a.out[(int64_t)m * a.ldo + c] = s_start;
+    }
+    float av, bv;
+    mingru_ab(a, m, c, s_start, av, bv);
+    A *= av;
+    B = av * B + bv;
+  }
+  a.ws[((int64_t)ch * 2) * a.n + c] = A;
+  a.ws[((int64_t)ch * 2 + 1) * a.n + c] = B;
+}
+
+__global__ __launch_bounds__(256) void mingru_pass2_kernel(MinGruArgs a, int n_chunks) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= a.n) return;
+  float S = 0.f;
+  for (int ch = 0; ch < n_chunks; ++ch) {
+    const float A = a.ws[((int64_t)ch * 2) * a.n + c], B = a.ws[((int64_t)ch * 2 + 1) * a.n + c];
+    a.ws[((int64_t)ch * 2) * a.n + c] = S;               // the chunk's carried-in state replaces its product
+    S = A * S + B;
+  }
+}
+
+__global__ __launch_bounds__(256) void mingru_pass3_kernel(MinGruArgs a) {
+  const int ch = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= a.n) return;
+  const int m0 = ch * MG_CH, m1 = min(a.M, m0 + MG_CH);
+  float S = a.ws[((int64_t)ch * 2) * a.n + c];
+  for (int m = m0; m < m1; ++m) {
+    const float s_start = a.row_back[m] == 0 ? a.out[(int64_t)m * a.ldo + c] : 0.f;
+    float av, bv;
+    mingru_ab(a, m, c, s_start, av, bv);
+    S = av * S + bv;
+    const float o = a.out_scale * S * silu_f(a.g[(int64_t)m * a.ldg + c]);
+    a.out[(int64_t)m * a.ldo + c] = o;
+    if (a.out16) a.out16[(int64_t)m * a.ldo16 + c] = f32_to_bf16(o);
+    if (m + 1 == a.M || a.row_back[m + 1] == 0) a.state[(int64_t)a.row_seq[m] * a.n + c] = S;
+  }
 }
 
 // one wave per row: `top` rounds of arg-max (ties: the lower index), then the softmax over the chosen logits.  Lane l owns the
@@ -505,6 +786,75 @@ extern "C" int mn_window_pool_attn(const float* q, int64_t ldq, const float* k_a
   return MN_OK;
 }
 
+extern "C" int mn_window_attn_block_rows(void) { return 4; }
+
+namespace {
+struct AttnShape { int aq, rows, hpc, chunks; };
+AttnShape attn_shape(int H, int G, int one_row) {
+  AttnShape s;
+  const int rep = H / G;
+  s.rows = one_row ? 1 : 4;
+  s.aq = (one_row && rep <= 4) ? 4 : 16;
+  s.hpc = s.aq / s.rows;
+  s.chunks = (rep + s.hpc - 1) / s.hpc;
+  return s;
+}
+}  // namespace
+
+extern "C" int mn_window_attn_splits(int n_blk, int H, int G, int one_row, int max_keys) {
+  if (n_blk < 1 || H < 1 || G < 1 || (H % G) != 0 || max_keys < 1) return 1;
+  const AttnShape sh = attn_shape(H, G, one_row);
+  const int64_t wgs = (int64_t)n_blk * G * sh.chunks, tiles = mn_cdiv(max_keys, AKT);
+  int64_t ns = mn_cdiv(2 * (int64_t)mn_num_cus(), wgs);
+  if (ns > tiles) ns = tiles;
+  if (ns > 64) ns = 64;
+  return ns < 1 ? 1 : (int)ns;
+}
+
+extern "C" size_t mn_window_attn_workspace_bytes(int n_blk, int H, int G, int vdim, int one_row, int nsplit) {
+  if (nsplit <= 1 || n_blk < 1 || H < 1 || G < 1 || (H % G) != 0) return 0;
+  const AttnShape sh = attn_shape(H, G, one_row);
+  return (size_t)n_blk * G * sh.chunks * nsplit * sh.aq * (2 + (size_t)vdim) * sizeof(float);
+}
+
+extern "C" int mn_window_pool_attn_blocks(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk,
+                                          const float* pv, const int32_t* row_seq, const int32_t* row_slot, const int32_t* blk_tab, int n_blk,
+                                          int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
+                                          float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  MN_CHECK_ARG(q && k_arena && v_arena && row_seq && row_slot && (out || out16) && n_blk >= 1 && H >= 1 && G >= 1 && (H % G) == 0 && dim >= 1 &&
+                   vdim >= 1 && vdim <= 512 && t_max >= 1 && window >= 0 && pool >= 0 && nsplit >= 1 && nsplit <= 65535,
+               "mn_window_pool_attn_blocks: bad args (vdim=%d: at most 512)", vdim);
+  MN_CHECK_ARG(pool == 0 || (window > 0 && pk && pv && n_pool_max >= 1), "mn_window_pool_attn_blocks: pooled blocks need a window and their arenas");
+  MN_CHECK_ARG(one_row || blk_tab, "mn_window_pool_attn_blocks: runs of several rows need their table");
+  const AttnShape sh = attn_shape(H, G, one_row);
+  MN_CHECK_ARG((int64_t)G * sh.chunks <= 65535, "mn_window_pool_attn_blocks: too many heads");
+  MN_CHECK_ARG(nsplit == 1 || (workspace && workspace_bytes >= mn_window_attn_workspace_bytes(n_blk, H, G, vdim, one_row, nsplit)),
+               "mn_window_pool_attn_blocks: workspace too small");
+  const size_t lds = ((size_t)sh.aq * dim + 2 * (size_t)sh.aq * AKT + 3 * sh.aq + (size_t)sh.aq * 256) * sizeof(float);
+  MN_CHECK_ARG(lds <= 64 * 1024, "mn_window_pool_attn_blocks: dim=%d too large", dim);
+  AttnTArgs a{q, ldq, k_arena, v_arena, pool ? pk : nullptr, pool ? pv : nullptr, row_seq, row_slot, one_row ? nullptr : blk_tab, H, G, dim, vdim,
+              t_max, n_pool_max, window, pool, sh.rows, sh.hpc, nsplit, out_scale, out, ldo, out16, ldo16, (float*)workspace};
+  const bool vec = (dim % 4) == 0 && (ldq % 4) == 0 && (((uintptr_t)q | (uintptr_t)k_arena | (uintptr_t)pk) & 15) == 0;
+  const dim3 grid((unsigned)n_blk, (unsigned)(G * sh.chunks), (unsigned)nsplit);
+  hipStream_t st = mn_stream(stream);
+  if (sh.aq == 4) {
+    if (vec) hipLaunchKernelGGL((window_attn_tiled_kernel<4, true>), grid, dim3(256), lds, st, a);
+    else hipLaunchKernelGGL((window_attn_tiled_kernel<4, false>), grid, dim3(256), lds, st, a);
+  } else {
+    if (vec) hipLaunchKernelGGL((window_attn_tiled_kernel<16, true>), grid, dim3(256), lds, st, a);
+    else hipLaunchKernelGGL((window_attn_tiled_kernel<16, false>), grid, dim3(256), lds, st, a);
+  }
+  MN_CHECK_LAUNCH("mn_window_pool_attn_blocks");
+  if (nsplit > 1) {
+    const dim3 mg((unsigned)n_blk, (unsigned)(G * sh.chunks));
+    if (sh.aq == 4) hipLaunchKernelGGL((window_attn_merge_kernel<4>), mg, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((window_attn_merge_kernel<16>), mg, dim3(256), 0, st, a);
+    MN_CHECK_LAUNCH("mn_window_pool_attn_blocks(merge)");
+  }
+  return MN_OK;
+}
+
 extern "C" int mn_mingru_rows(const float* zx, int64_t ldzx, const float* g, int64_t ldg, float* state, const int32_t* row_seq,
                               const int32_t* row_slot, const int32_t* row_back, float out_scale, float* out, int64_t ldo, uint16_t* out16,
                               int64_t ldo16, int M, int n, void* stream) {
@@ -513,6 +863,27 @@ extern "C" int mn_mingru_rows(const float* zx, int64_t ldzx, const float* g, int
   hipLaunchKernelGGL(mingru_kernel, dim3((unsigned)mn_cdiv(n, 256), (unsigned)M), dim3(256), 0, mn_stream(stream), zx, ldzx, g, ldg, state,
                      row_seq, row_slot, row_back, out_scale, out, ldo, out16, ldo16, M, n);
   MN_CHECK_LAUNCH("mn_mingru_rows");
+  return MN_OK;
+}
+
+extern "C" size_t mn_mingru_scan_workspace_bytes(int M, int n) {
+  return M < 1 || n < 1 ? 0 : (size_t)mn_cdiv(M, MG_CH) * 2 * n * sizeof(float);
+}
+
+extern "C" int mn_mingru_rows_scan(const float* zx, int64_t ldzx, const float* g, int64_t ldg, float* state, const int32_t* row_seq,
+                                   const int32_t* row_slot, const int32_t* row_back, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                                   int64_t ldo16, int M, int n, void* workspace, size_t workspace_bytes, void* stream) {
+  MN_CHECK_ARG(zx && g && state && row_seq && row_slot && row_back && out && M >= 1 && n >= 1 && mn_cdiv(M, MG_CH) <= 65535,
+               "mn_mingru_rows_scan: bad args");
+  MN_CHECK_ARG(workspace && workspace_bytes >= mn_mingru_scan_workspace_bytes(M, n), "mn_mingru_rows_scan: workspace too small");
+  MinGruArgs a{zx, ldzx, g, ldg, state, row_seq, row_slot, row_back, out_scale, out, ldo, out16, ldo16, (float*)workspace, M, n};
+  const int n_chunks = (int)mn_cdiv(M, MG_CH);
+  const dim3 grid((unsigned)mn_cdiv(n, 256), (unsigned)n_chunks);
+  hipStream_t st = mn_stream(stream);
+  hipLaunchKernelGGL(mingru_pass1_kernel, grid, dim3(256), 0, st, a);
+  hipLaunchKernelGGL(mingru_pass2_kernel, dim3(grid.x), dim3(256), 0, st, a, n_chunks);
+  hipLaunchKernelGGL(mingru_pass3_kernel, grid, dim3(256), 0, st, a);
+  MN_CHECK_LAUNCH("mn_mingru_rows_scan");
   return MN_OK;
 }
 

@@ -1,4 +1,5 @@
-"""Prefill / decode throughput of the Pizitar decoder beside the Bailing-MoE decoder at equal size (`bench.py --lm-compare`).
+"""Prefill / decode throughput of the Pizitar or the Sakinex decoder beside the Bailing-MoE decoder at equal size
+(`bench.py --lm-compare [--lm-model sakinex]`).
 
 Random weights at sizes that resemble real layers.  "Equal size": same width, depth and head count, 128-wide heads on both, and a
 feed-forward whose ACTIVE hidden width matches (the MoE runs 8 experts, top-2, of half the dense hidden width each).  Both run
@@ -7,6 +8,13 @@ Beside the end-to-end rates the attention kernels are timed alone against their 
   decode   bytes of cache read per step / HBM peak        (latents [len, r] fp32  vs  keys + values [len, n_kv, 128] x 2 fp32)
   prefill  multiply-adds of the causal score / value products at the precision the kernel runs them
            (fp32 FMA peak for the latent kernel, bf16 MFMA peak for the flash kernel)
+
+Sakinex at "equal size": same width, depth, query / key-value head counts and 128-wide heads as the Bailing-MoE side, the same 8
+experts, top-2, plus one shared expert on both, a recurrence as wide as the model, a window of 1024 tokens with pooled blocks of 16,
+no repeated layers.  Its attention reads at most window + length / pool keys per row, so its rooflines are priced on THOSE keys:
+  decode   bytes of the visible keys and values (token arenas + block-mean arenas) per step / HBM peak
+  prefill  multiply-adds of the visible score / value products on the fp32 FMA peak (the kernel's arithmetic)
+and the recurrence alone on the bytes it reads and writes.
 """
 import time
 
@@ -43,11 +51,23 @@ def pizitar_config(s):
                          logit_softcap=30.0)
 
 
-def bailing_config(s):
+def sakinex_config(s):
+    from .configuration import SakinexConfig
+    left = dict(conv=4, dim=128, vdim=128, heads=s["heads"], kv_heads=s["heads"] // 4, mask=dict(pool=SAKINEX_POOL, size=SAKINEX_WINDOW),
+                rot=dict(base=600000.0, dims=128, scaling=dict(factor=8.0, fast=32.0, original=4096, slow=1.0)), scale=128 ** -0.5)
+    ly = dict(type="parallel", mixer=dict(left=left, left_scale=0.7, right=dict(width=s["width"]), right_scale=0.7),
+              mlp=dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=s["ff"] // 2), shared=dict(ff=s["ff"] // 2)))
+    return SakinexConfig(width=s["width"], vocab=s["vocab"], layers=[ly] * s["layers"], canon=dict(taps=4), norm=dict(eps=1e-6), residual_mult=0.5)
+
+
+SAKINEX_WINDOW, SAKINEX_POOL = 1024, 16
+
+
+def bailing_config(s, shared=0):
     from .configuration import BailingMoeConfig
     return BailingMoeConfig(vocab_size=s["vocab"], hidden_size=s["width"], num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
                             num_key_value_heads=s["heads"] // 4, head_dim=128, use_bias=False, use_qkv_bias=False, rope_theta=600000.0,
-                            num_experts=8, num_shared_experts=0, num_experts_per_tok=2, moe_intermediate_size=s["ff"] // 2, multi_gate=False,
+                            num_experts=8, num_shared_experts=shared, num_experts_per_tok=2, moe_intermediate_size=s["ff"] // 2, multi_gate=False,
                             first_k_dense_replace=0, norm_topk_prob=True)
 
 
@@ -112,12 +132,81 @@ def run_pizitar(s, T, batches, n_dec):
     return out
 
 
-def run_bailing(s, T, batches, n_dec):
+def run_sakinex(s, T, batches, n_dec):
+    from ._lib import check, current_stream, lib, ptr
+    from .sakinex import SakinexDecoder
+    from .sequences import rows_of_spans
+    dev = "cuda"
+    cfg = sakinex_config(s)
+    dec = SakinexDecoder.synthetic(cfg, dev, t_max=T + n_dec + 8, n_seq=max(batches), arith="bf16")
+    ids = torch.randint(0, s["vocab"], (T,), device=dev)
+    x = dec.embed(ids)
+    out = {"prefill_tokens_per_s": T / _time(lambda: dec.forward_spans(x, [(0, T, 0)]), 3)}
+    for B in batches:
+        for run in dec.state_t:                              # every sequence continues the prompt of sequence 0
+            for k, t in run.items():
+                if t is not None:
+                    ax = dec.SEQ_AXIS[k]
+                    t.narrow(ax, 1, B - 1).copy_(t.narrow(ax, 0, 1).expand_as(t.narrow(ax, 1, B - 1))) if B > 1 else None
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        back, blk = dec.decode_tables(B)
+        xb = dec.embed(torch.randint(0, s["vocab"], (B,), device=dev))
+
+        def loop():
+            slot = torch.full((B,), T, dtype=torch.int32, device=dev)
+            ln = slot + 1
+            for i in range(n_dec):
+                dec.step(xb, row_seq, slot, back, ln, blk, T + i + 1, distinct=True)
+                check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
+        out[f"decode_b{B}_tokens_per_s"] = B * n_dec / _time(loop, 2, 1)
+        slot_g = torch.full((B,), T, dtype=torch.int32, device=dev)
+        ln_g = slot_g + 1
+        graph = dec.decode_graph(row_seq, slot_g, ln_g)
+
+        def loop_graph():
+            slot_g.fill_(T)
+            ln_g.fill_(T + 1)
+            for i in range(n_dec):
+                graph.run(xb, T + i + 1)
+        out[f"decode_b{B}_graph_tokens_per_s"] = B * n_dec / _time(loop_graph, 2, 1)
+    # the attention kernel alone, on the first run's arenas
+    H, G, d = s["heads"], s["heads"] // 4, 128
+    st = dec.state_t[0]
+    tabs = {k: torch.from_numpy(v).to(dev) for k, v in rows_of_spans([(0, T, 0)], 1 << 30).items() if k != "max_len"}
+    q = torch.randn(T, H * d, device=dev) * 0.05
+    att = torch.empty(T, H * d, device=dev)
+
+    def attn(M, rs, rp):
+        check(lib().mn_window_pool_attn(ptr(q), H * d, ptr(st["k"]), ptr(st["v"]), ptr(st["pk"]), ptr(st["pv"]), ptr(rs), ptr(rp), M, H, G, d, d,
+                                        dec.t_max, dec.n_pool_max, SAKINEX_WINDOW, SAKINEX_POOL, 1.0, ptr(att), H * d, None, 0, current_stream()),
+              "mn_window_pool_attn")
+
+    def keys_at(i):
+        return min(i + 1, SAKINEX_WINDOW) + max(0, (i - SAKINEX_WINDOW + 1) // SAKINEX_POOL)
+    t = _time(lambda: attn(T, tabs["row_seq"], tabs["row_slot"]), 5)
+    flops = 2 * 2 * H * d * sum(keys_at(i) for i in range(T))
+    out["attn_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / FMA_F32_TFLOPS, peak="fp32 FMA")
+    for B in batches:
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        slot = torch.full((B,), T - 1, dtype=torch.int32, device=dev)
+        t = _time(lambda: attn(B, row_seq, slot), 20)
+        byts = B * keys_at(T - 1) * G * 2 * d * 4
+        out[f"attn_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS, keys=keys_at(T - 1))
+    # the recurrence alone: reads z, u, g, writes the gated state (fp32 rows)
+    n = s["width"]
+    zx, gg, o = torch.randn(T, 2 * n, device=dev), torch.randn(T, n, device=dev), torch.empty(T, n, device=dev)
+    t = _time(lambda: check(lib().mn_mingru_rows(ptr(zx), 2 * n, ptr(gg), n, ptr(st["gru"]), ptr(tabs["row_seq"]), ptr(tabs["row_slot"]),
+                                                 ptr(tabs["row_back"]), 1.0, ptr(o), n, None, 0, T, n, current_stream()), "mn_mingru_rows"), 5)
+    out["mingru_prefill"] = dict(us=t * 1e6, gbs=T * n * 16 / t / 1e9, of_peak=T * n * 16 / t / 1e9 / HBM_GBS)
+    return out
+
+
+def run_bailing(s, T, batches, n_dec, shared=0):
     from . import ops
     from ._lib import check, current_stream, lib, ptr
     from .bailing_moe import BailingMoeDecoder
     dev = "cuda"
-    cfg = bailing_config(s)
+    cfg = bailing_config(s, shared)
     dec = BailingMoeDecoder.synthetic(cfg, dev, t_max=T + n_dec + 8, n_seq=max(batches))
     ids = torch.randint(0, s["vocab"], (T,), device=dev)
     x = dec.embed(ids)
@@ -156,12 +245,15 @@ def run_bailing(s, T, batches, n_dec):
     return out
 
 
-def compare(sizes=("w1024", "w2048"), prompt=2048, batches=(1, 32), n_dec=32):
+def compare(sizes=("w1024", "w2048"), prompt=2048, batches=(1, 32), n_dec=32, model="pizitar"):
     res = {}
     for name in sizes:
         s = SIZES[name]
         torch.cuda.empty_cache()
-        res[name] = dict(size=s, prompt=prompt, pizitar=run_pizitar(s, prompt, batches, n_dec))
+        if model == "sakinex":
+            res[name] = dict(size=s, prompt=prompt, sakinex=run_sakinex(s, prompt, batches, n_dec))
+        else:
+            res[name] = dict(size=s, prompt=prompt, pizitar=run_pizitar(s, prompt, batches, n_dec))
         torch.cuda.empty_cache()
-        res[name]["bailing_moe"] = run_bailing(s, prompt, batches, n_dec)
+        res[name]["bailing_moe"] = run_bailing(s, prompt, batches, n_dec, shared=1 if model == "sakinex" else 0)
     return res

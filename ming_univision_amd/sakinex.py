@@ -127,7 +127,7 @@ class SakinexDecoder(SeqDecoder):
         self.n_pool_max = self.t_max // min(pools) + 1 if pools else 1
         self.state_t = self._alloc_state(self.n_seq)
         self._bind_state()
-        self.block_rows = 1 << 30                        # the attention takes rows one by one: no row blocks to cut
+        self.block_rows = int(lib().mn_window_attn_block_rows())
         self._ws, self._decode_tabs = {}, {}
 
     def _p(self, t):
@@ -237,8 +237,9 @@ class SakinexDecoder(SeqDecoder):
 
     def step(self, x, row_seq, row_slot, row_back, row_len=None, blk_tab=None, max_len=None, out=None, trace=None, ws=None, distinct=False):
         """One pass of the stack over M rows.  x fp32 [M, width] (input embeddings); int32 device arrays per row (row r is position
-        row_slot[r] of cache sequence row_seq[r], preceded in this pass by row_back[r] rows of its sequence).  row_len / blk_tab are
-        the other decoder's per-row tables and are not read here; max_len (host int) >= every position + 1.  Appends the rows' keys
+        row_slot[r] of cache sequence row_seq[r], preceded in this pass by row_back[r] rows of its sequence); blk_tab int32 [n_blk, 2]
+        cuts the rows into runs of <= block_rows consecutive rows of one sequence (not read when distinct); row_len is the other
+        decoder's table and is not read here; max_len (host int) >= every position + 1 (default: the cache's length).  Appends the rows' keys
         and values, completes pooled blocks, advances the filter and recurrent states.  trace: optional fp32 [runs, M, width] that
         receives the residual stream after every layer run.  distinct: every row is alone in its sequence (a decode step): the step
         fuses its residual add / norm / filter launches.  Returns the final norm's output [M, width] fp32."""
@@ -246,7 +247,10 @@ class SakinexDecoder(SeqDecoder):
         assert x.dtype == torch.float32 and x.is_cuda and x.stride(1) == 1 and x.shape[1] == self.cfg.width and 1 <= M <= self.max_rows()
         for t in (row_seq, row_slot, row_back):
             assert t.dtype == torch.int32 and t.is_cuda and t.is_contiguous() and t.numel() >= M
-        assert max_len is None or 1 <= max_len <= self.t_max, f"{max_len} tokens exceed the cache (t_max = {self.t_max})"
+        max_len = self.t_max if max_len is None else int(max_len)
+        assert 1 <= max_len <= self.t_max, f"{max_len} tokens exceed the cache (t_max = {self.t_max})"
+        if not distinct:
+            assert blk_tab is not None and blk_tab.dtype == torch.int32 and blk_tab.is_cuda and blk_tab.is_contiguous() and blk_tab.shape[1] == 2
         if out is None:
             out = torch.empty(M, self.cfg.width, dtype=torch.float32, device=self.device)
         if trace is not None:
@@ -254,7 +258,8 @@ class SakinexDecoder(SeqDecoder):
         if ws is None:
             ws = self._workspace(M, max_len)
         check(lib().mn_pmix_step(C.byref(self.struct), C.byref(self.state), ptr(x), x.stride(0), M, ptr(row_seq), ptr(row_slot), ptr(row_back),
-                                 1 if distinct else 0, ptr(out), ptr(trace), ptr(ws), ws.numel(), current_stream()), "mn_pmix_step")
+                                 None if distinct else ptr(blk_tab), M if distinct else blk_tab.shape[0], max_len, 1 if distinct else 0, ptr(out),
+                                 ptr(trace), ptr(ws), ws.numel(), current_stream()), "mn_pmix_step")
         return out
 
 

@@ -234,6 +234,29 @@ def _attention_case(T, H, G, dim, vdim, window, pool, peaky, seed, rows=None):
                                 len(rows), H, G, dim, vdim, t_max, npm, window, pool, 0.6, ptr(out), H * vdim + 5, ptr(out16), H * vdim, stream()))
     assert err(out[:, :H * vdim], 0.6 * ref[sel]) < 2e-5
     assert err(out16.float(), 0.6 * ref[sel]) < 1e-2
+    # the tiled form: single rows with several key splits, then runs of up to block_rows consecutive rows
+    from ming_univision_amd.sequences import rows_of_spans
+    for nsplit in (1, 3, 64):
+        out.fill_(float("nan"))
+        ws = torch.empty(max(16, L.mn_window_attn_workspace_bytes(len(rows), H, G, vdim, 1, nsplit)), dtype=torch.uint8, device="cuda")
+        check(L.mn_window_pool_attn_blocks(ptr(qd), H * dim, ptr(ka), ptr(va), ptr(pk) if pool else None, ptr(pv) if pool else None, ptr(rs), ptr(rp),
+                                           None, len(rows), 1, H, G, dim, vdim, t_max, npm, window, pool, 0.6, ptr(out), H * vdim + 5, ptr(out16),
+                                           H * vdim, nsplit, ptr(ws), ws.numel(), stream()))
+        assert err(out[:, :H * vdim], 0.6 * ref[sel]) < 2e-5, nsplit
+        assert err(out16.float(), 0.6 * ref[sel]) < 1e-2
+    if len(rows) == T:
+        RB = L.mn_window_attn_block_rows()
+        for past in (0, 3):                                   # runs that start at position 0, and runs that straddle block and window edges otherwise
+            spans = [(1, past, 0), (1, T - past, past)] if past else [(1, T, 0)]
+            tb = rows_of_spans(spans, RB)
+            blk = torch.from_numpy(tb["blk_tab"]).cuda()
+            for nsplit in (1, 2):
+                outb = torch.full((T, H * vdim), float("nan"), device="cuda")
+                ws = torch.empty(max(16, L.mn_window_attn_workspace_bytes(blk.shape[0], H, G, vdim, 0, nsplit)), dtype=torch.uint8, device="cuda")
+                check(L.mn_window_pool_attn_blocks(ptr(qd), H * dim, ptr(ka), ptr(va), ptr(pk) if pool else None, ptr(pv) if pool else None,
+                                                   ptr(r["row_seq"]), ptr(r["row_slot"]), ptr(blk), blk.shape[0], 0, H, G, dim, vdim, t_max, npm, window,
+                                                   pool, 0.6, ptr(outb), H * vdim, None, 0, nsplit, ptr(ws), ws.numel(), stream()))
+                assert err(outb, 0.6 * ref) < 2e-5, (past, nsplit)
 
 
 @pytest.mark.parametrize("H,G,dim,vdim,window,pool", [(4, 2, 16, 24, 9, 4), (3, 1, 12, 20, 7, 3), (2, 2, 16, 16, 1, 1), (12, 1, 8, 8, 0, 0),
@@ -278,6 +301,32 @@ def test_min_gru_rows_carry_their_state():
     check(L.mn_mingru_rows(ptr(D(torch.cat([zx[:4], zx[:3]]))), zx.shape[1], ptr(D(torch.cat([gg[:4], gg[:3]]))), n, ptr(state), ptr(r["row_seq"]),
                            ptr(r["row_slot"]), ptr(r["row_back"]), 0.5, ptr(out), n, None, 0, 7, n, stream()))
     assert err(out[:4], ref[:4]) < 1e-5 and err(out[4:], ref[:3]) < 1e-5
+    # the chunked scan: a sequence that continues from its state, one that starts, one of a single row, chunk edges inside them
+    zx2, gg2 = torch.randn(150, 2 * n + 3, generator=g) * 2, torch.randn(150, n, generator=g)
+    st0 = torch.randn(4, n, generator=g)
+    spans = [(3, 70, 5), (0, 1, 0), (1, 47, 0), (2, 32, 9)]
+    want, fin, at = [], {}, 0
+    for seq, cnt, past in spans:
+        S = st0[seq].double() if past else torch.zeros(n, dtype=torch.float64)
+        for t in range(at, at + cnt):
+            z, c = torch.sigmoid(zx2[t, :n].double()), O.gru_candidate(zx2[t, n:2 * n].double())
+            S = (1 - z) * S + z * c
+            want.append(0.5 * S * gg2[t].double() * torch.sigmoid(gg2[t].double()))
+        fin[seq], at = S, at + cnt
+    r = _rows(spans)
+    for scan in (True, False):
+        std, out = st0.cuda(), torch.empty(150, n + 2, device="cuda")
+        o16 = torch.empty(150, n, dtype=torch.bfloat16, device="cuda")
+        if scan:
+            ws = torch.empty(L.mn_mingru_scan_workspace_bytes(150, n), dtype=torch.uint8, device="cuda")
+            check(L.mn_mingru_rows_scan(ptr(D(zx2)), zx2.shape[1], ptr(D(gg2)), n, ptr(std), ptr(r["row_seq"]), ptr(r["row_slot"]), ptr(r["row_back"]), 0.5,
+                                        ptr(out), n + 2, ptr(o16), n, 150, n, ptr(ws), ws.numel(), stream()))
+        else:
+            check(L.mn_mingru_rows(ptr(D(zx2)), zx2.shape[1], ptr(D(gg2)), n, ptr(std), ptr(r["row_seq"]), ptr(r["row_slot"]), ptr(r["row_back"]), 0.5,
+                                   ptr(out), n + 2, ptr(o16), n, 150, n, stream()))
+        assert err(out[:, :n], torch.stack(want)) < 1e-5 and err(o16.float(), torch.stack(want)) < 1e-2, scan
+        for seq in fin:
+            assert err(std[seq], fin[seq]) < 1e-5, (scan, seq)
 
 
 def test_router_and_expert_operators():
@@ -319,7 +368,7 @@ def test_router_and_expert_operators():
 @pytest.mark.parametrize("name", list(MODELS))
 def test_prompt_layers_and_logits(name):
     cfg, sd, dec = make(name)
-    t = toks(cfg, 60)
+    t = toks(cfg, 81)                                     # above 64 rows: the recurrence runs as a chunked scan
     ref, streams = O.forward(cfg, sd, t, trace=True)
     hid, tr = dec.forward_spans(dec.embed(torch.tensor(t, device="cuda")), [(0, len(t), 0)], trace=True)
     assert tr.shape[0] == len(O.layer_runs(cfg))
