@@ -1,7 +1,10 @@
 // pmix_engine.hip — the step function of parallel-mixer sequence models (mingnative.h section 10): one pass of the layer runs over
 // the rows of a step as a chain of launches on the caller's stream.  Matrix products go through the routing of seq_linear.h; the
 // experts of a mixture-of-experts feed-forward run
-//   MN_SEQ_ARITH_BF16, M > 64   sorted by expert on the grouped bf16 MFMA GEMM (mn_moe_sort, mn_gather_rows_bf16, mn_gemm_bf16_grouped)
+//   MN_SEQ_ARITH_BF16, M > 8    sorted by expert on a grouped bf16 MFMA GEMM: the 256 x 256-tile kernel over the list of live row tiles
+//                               (mn_moe_sort_tiles, mn_gemm256_grouped_tiles: rows gathered while staging, SwiGLU in the gate / up
+//                               epilogue) when width and expert width are multiples of 64, else the 128-tile kernel
+//                               (mn_moe_sort, mn_gather_rows_bf16, mn_gemm_bf16_grouped) when they are multiples of 8
 //   otherwise                   one (row, pick) pair at a time against the weights its index names (mn_gemv_f32_indexed, fp32 FMA)
 #include "seq_linear.h"
 
@@ -30,9 +33,16 @@ struct PPlan {
   size_t gemm_ws = 0, attn_ws = 0, gru_ws = 0;
 };
 
-bool grouped_route(const mn_pmix_model* m, const mn_pmix_layer& l, int M) {
-  return m->arith == MN_SEQ_ARITH_BF16 && M > 64 && l.experts <= 128 && (int64_t)M * l.top <= 65536 && (m->width % 8) == 0 &&
-         (l.ff % 8) == 0 && ((((uintptr_t)l.w_gate_up) | ((uintptr_t)l.w_down)) & 15) == 0;
+enum { EXPERTS_INDEXED = 0, EXPERTS_GROUPED = 1, EXPERTS_TILES = 2 };
+int expert_route(const mn_pmix_model* m, const mn_pmix_layer& l, int M) {
+  if (m->arith != MN_SEQ_ARITH_BF16 || M <= 8 || l.experts > 128 || (int64_t)M * l.top > 65536 ||
+      ((((uintptr_t)l.w_gate_up) | ((uintptr_t)l.w_down)) & 15) != 0)
+    return EXPERTS_INDEXED;
+  const int64_t W = m->width, ff = l.ff;
+  if ((W % 64) == 0 && (ff % 64) == 0 && 2 * ff * W * 2 < ((int64_t)1 << 32) && (int64_t)M * l.top * (W > ff ? W : ff) * 2 < ((int64_t)1 << 32))
+    return EXPERTS_TILES;
+  if ((W % 8) == 0 && (ff % 8) == 0) return EXPERTS_GROUPED;
+  return EXPERTS_INDEXED;
 }
 
 PPlan make_plan(const mn_pmix_model* m, int M) {
@@ -91,6 +101,7 @@ extern "C" size_t mn_pmix_workspace_bytes(const mn_pmix_model* m, int M) {
   n += al(Z * W * 4);                                  // their results
   n += al(Z * W * 2);                                  // gathered bf16 rows
   n += 2 * al(((size_t)p.experts + 1) * 4) + 2 * al(Z * 4);   // counts, offsets, perm, slot_of
+  n += 2 * al((Z / 256 + p.experts + 1) * 4) + al(4);         // live row tiles of the grouped products, their count
   n += al(p.gemm_ws) + al(p.attn_ws) + al(p.gru_ws);
   return n;
 }
@@ -140,6 +151,10 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
   int32_t* offsets = (int32_t*)take(((size_t)p.experts + 1) * 4);
   int32_t* perm = (int32_t*)take(Zmax * 4);
   int32_t* slot_of = (int32_t*)take(Zmax * 4);
+  int32_t* tile_g = (int32_t*)take((Zmax / 256 + p.experts + 1) * 4);
+  int32_t* tile_m0 = (int32_t*)take((Zmax / 256 + p.experts + 1) * 4);
+  int32_t* n_tiles = (int32_t*)take(4);
+  uint16_t* const hh_buf = hh;
   void* gws = p.gemm_ws ? take(p.gemm_ws) : nullptr;
   const size_t gwb = p.gemm_ws;
   void* aws = take(p.attn_ws);
@@ -246,7 +261,20 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
         MN_TRY(linear(arith, M, sa, fs, sah, fs, l.w_shared_down, W, fs, nullptr, sh, W, gws, gwb, stream));
       }
       const int32_t* so = nullptr;
-      if (h16 && grouped_route(m, l, M)) {
+      const int route = expert_route(m, l, M);
+      if (route != EXPERTS_INDEXED && !h16) {          // few rows: the sublayer input was written in fp32 only
+        MN_TRY(mn_f32_to_bf16(h, hh_buf, (int64_t)M * W, stream));
+        h16 = hh_buf;
+      }
+      if (route == EXPERTS_TILES) {
+        const int max_mtiles = Z / 256 + E;
+        MN_TRY(mn_moe_sort_tiles(tidx, M, top, E, counts, offsets, perm, slot_of, 256, tile_g, tile_m0, n_tiles, stream));
+        MN_TRY(mn_gemm256_grouped_tiles(h16, W, 0, M, perm, l.w_gate_up, W, (int64_t)2 * ff * W, offsets, counts, E, tile_g, tile_m0, n_tiles,
+                                        max_mtiles, eah, ff, 0, ff, W, 6, stream));
+        MN_TRY(mn_gemm256_grouped_tiles(eah, ff, 0, Z, nullptr, l.w_down, ff, (int64_t)W * ff, offsets, counts, E, tile_g, tile_m0, n_tiles,
+                                        max_mtiles, ye, W, 0, W, ff, 0, stream));
+        so = slot_of;
+      } else if (route == EXPERTS_GROUPED) {
         MN_TRY(mn_moe_sort(tidx, M, top, E, counts, offsets, perm, slot_of, stream));
         MN_TRY(mn_gather_rows_bf16(h16, W, perm, xg, W, Z, W, stream));
         MN_TRY(mn_gemm_bf16_grouped(xg, W, l.w_gate_up, W, (int64_t)2 * ff * W, offsets, counts, E, gu, 2 * ff, M, 2 * ff, W, MN_GEMM_F32, stream));

@@ -385,6 +385,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
   const float* pkb = a.pk ? a.pk + (int64_t)seq * a.n_pool_max * Gd + (int64_t)g * a.dim : nullptr;
   const float* pvb = a.pv ? a.pv + (int64_t)seq * a.n_pool_max * Gv + (int64_t)g * a.vdim : nullptr;
   constexpr int NCB = 2;                    // column blocks of 256: vdim <= 512
+  constexpr int PRE = AQ == 4 ? 8 : 2;      // loads in flight per thread: deep for the few vectors of decode rows, where latency is all there is
   float acc[NCB][AQ];
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb)
@@ -402,12 +403,23 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
       for (int i = 0; i < AQ; ++i) s[i] = 0.f;
       if (valid) {
         if (VEC) {
-          for (int f = part; f < a.dim / 4; f += 4) {
-            const float4 kv = *reinterpret_cast<const float4*>(kp + 4 * f);
+          const int nf = a.dim / 4;
+          for (int f0 = part; f0 < nf; f0 += 4 * PRE) {   // PRE 16-byte pieces of the key in flight before the first product
+            float4 kv[PRE];
 #pragma unroll
-            for (int i = 0; i < AQ; ++i) {
-              const float4 qq = *reinterpret_cast<const float4*>(qs + i * a.dim + 4 * f);
-              s[i] = fmaf(qq.x, kv.x, s[i]); s[i] = fmaf(qq.y, kv.y, s[i]); s[i] = fmaf(qq.z, kv.z, s[i]); s[i] = fmaf(qq.w, kv.w, s[i]);
+            for (int u = 0; u < PRE; ++u) {
+              const int f = f0 + 4 * u;
+              kv[u] = f < nf ? *reinterpret_cast<const float4*>(kp + 4 * f) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int u = 0; u < PRE; ++u) {
+              const int f = f0 + 4 * u;
+              if (f >= nf) break;
+#pragma unroll
+              for (int i = 0; i < AQ; ++i) {
+                const float4 qq = *reinterpret_cast<const float4*>(qs + i * a.dim + 4 * f);
+                s[i] = fmaf(qq.x, kv[u].x, s[i]); s[i] = fmaf(qq.y, kv[u].y, s[i]); s[i] = fmaf(qq.z, kv[u].z, s[i]); s[i] = fmaf(qq.w, kv[u].w, s[i]);
+              }
             }
           }
         } else {
@@ -457,15 +469,24 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
       if (ksub < nsub) {
 #pragma unroll
         for (int i = 0; i < AQ; ++i) acc[cb][i] *= st_a[i];
-        for (int jj = ksub; jj < nt; jj += nsub) {
-          const int j = j0 + jj;
-          const float vv = (j < nbL ? pvb + (int64_t)j * Gv : vb + (int64_t)(j - nbL) * Gv)[c0 + c];
-          const float* pr = pT + jj * AQ;
+        for (int jj0 = ksub; jj0 < nt; jj0 += PRE * nsub) {  // PRE values of the column in flight before the first product
+          float vv[PRE];
 #pragma unroll
-          for (int i = 0; i < AQ; i += 4) {
-            const float4 pp = *reinterpret_cast<const float4*>(pr + i);
-            acc[cb][i] = fmaf(pp.x, vv, acc[cb][i]); acc[cb][i + 1] = fmaf(pp.y, vv, acc[cb][i + 1]);
-            acc[cb][i + 2] = fmaf(pp.z, vv, acc[cb][i + 2]); acc[cb][i + 3] = fmaf(pp.w, vv, acc[cb][i + 3]);
+          for (int u = 0; u < PRE; ++u) {
+            const int jj = jj0 + u * nsub, j = j0 + jj;
+            vv[u] = jj < nt ? (j < nbL ? pvb + (int64_t)j * Gv : vb + (int64_t)(j - nbL) * Gv)[c0 + c] : 0.f;
+          }
+#pragma unroll
+          for (int u = 0; u < PRE; ++u) {
+            const int jj = jj0 + u * nsub;
+            if (jj >= nt) break;
+            const float* pr = pT + jj * AQ;
+#pragma unroll
+            for (int i = 0; i < AQ; i += 4) {
+              const float4 pp = *reinterpret_cast<const float4*>(pr + i);
+              acc[cb][i] = fmaf(pp.x, vv[u], acc[cb][i]); acc[cb][i + 1] = fmaf(pp.y, vv[u], acc[cb][i + 1]);
+              acc[cb][i + 2] = fmaf(pp.z, vv[u], acc[cb][i + 2]); acc[cb][i + 3] = fmaf(pp.w, vv[u], acc[cb][i + 3]);
+            }
           }
         }
       }
@@ -515,18 +536,29 @@ __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
   const int nqv = nr * Rc;
   const int64_t stride = (int64_t)AQ * (2 + a.vdim);
   const float* base = a.part + ((int64_t)b * gridDim.y + gy) * a.nsplit * stride;
+  // the weight of every (vector, split) once per workgroup: exp(its maximum - the overall maximum), and the vectors' normalisers
+  __shared__ float wgt[AQ * 64];
+  __shared__ float Ls[AQ];
+  if (tid < AQ) {
+    float mx = -INFINITY;
+    for (int s = 0; s < a.nsplit; ++s) mx = fmaxf(mx, base[s * stride + tid]);
+    float L = 0.f;
+    for (int s = 0; s < a.nsplit; ++s) {
+      const float ms = base[s * stride + tid];
+      const float w = ms == -INFINITY ? 0.f : expf(ms - mx);
+      wgt[tid * 64 + s] = w;
+      L = fmaf(base[s * stride + AQ + tid], w, L);
+    }
+    Ls[tid] = L;
+  }
+  __syncthreads();
   for (int e = tid; e < nqv * a.vdim; e += 256) {
     const int i = e / a.vdim, c = e - i * a.vdim;
-    float mx = -INFINITY;
-    for (int s = 0; s < a.nsplit; ++s) mx = fmaxf(mx, base[s * stride + i]);
-    float L = 0.f, t = 0.f;
-    for (int s = 0; s < a.nsplit; ++s) {
-      const float ms = base[s * stride + i];
-      if (ms == -INFINITY) continue;
-      const float w = expf(ms - mx);
-      L = fmaf(base[s * stride + AQ + i], w, L);
-      t = fmaf(base[s * stride + 2 * AQ + (int64_t)i * a.vdim + c], w, t);
-    }
+    const float* src = base + 2 * AQ + (int64_t)i * a.vdim + c;
+    float t = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < a.nsplit; ++s) t = fmaf(src[s * stride], wgt[i * 64 + s], t);
+    const float L = Ls[i];
     const float val = t / L * a.out_scale;
     const int64_t col = (int64_t)(h0 + i % Rc) * a.vdim + c;
     const int row = r0 + i / Rc;
@@ -823,8 +855,8 @@ extern "C" int mn_window_pool_attn_blocks(const float* q, int64_t ldq, const flo
                                           float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
                                           size_t workspace_bytes, void* stream) {
   MN_CHECK_ARG(q && k_arena && v_arena && row_seq && row_slot && (out || out16) && n_blk >= 1 && H >= 1 && G >= 1 && (H % G) == 0 && dim >= 1 &&
-                   vdim >= 1 && vdim <= 512 && t_max >= 1 && window >= 0 && pool >= 0 && nsplit >= 1 && nsplit <= 65535,
-               "mn_window_pool_attn_blocks: bad args (vdim=%d: at most 512)", vdim);
+                   vdim >= 1 && vdim <= 512 && t_max >= 1 && window >= 0 && pool >= 0 && nsplit >= 1 && nsplit <= 64,
+               "mn_window_pool_attn_blocks: bad args (vdim=%d: at most 512; nsplit=%d: at most 64)", vdim, nsplit);
   MN_CHECK_ARG(pool == 0 || (window > 0 && pk && pv && n_pool_max >= 1), "mn_window_pool_attn_blocks: pooled blocks need a window and their arenas");
   MN_CHECK_ARG(one_row || blk_tab, "mn_window_pool_attn_blocks: runs of several rows need their table");
   const AttnShape sh = attn_shape(H, G, one_row);

@@ -176,27 +176,39 @@ def run_sakinex(s, T, batches, n_dec):
     q = torch.randn(T, H * d, device=dev) * 0.05
     att = torch.empty(T, H * d, device=dev)
 
-    def attn(M, rs, rp):
-        check(lib().mn_window_pool_attn(ptr(q), H * d, ptr(st["k"]), ptr(st["v"]), ptr(st["pk"]), ptr(st["pv"]), ptr(rs), ptr(rp), M, H, G, d, d,
-                                        dec.t_max, dec.n_pool_max, SAKINEX_WINDOW, SAKINEX_POOL, 1.0, ptr(att), H * d, None, 0, current_stream()),
-              "mn_window_pool_attn")
+    RB = lib().mn_window_attn_block_rows()
+    blk = torch.from_numpy(rows_of_spans([(0, T, 0)], RB)["blk_tab"]).to(dev)
+    aws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+
+    def attn(M, rs, rp, one_row):
+        n_blk = M if one_row else blk.shape[0]
+        keys = SAKINEX_WINDOW + (0 if one_row else RB - 1) + T // SAKINEX_POOL
+        ns = lib().mn_window_attn_splits(n_blk, H, G, one_row, keys)
+        check(lib().mn_window_pool_attn_blocks(ptr(q), H * d, ptr(st["k"]), ptr(st["v"]), ptr(st["pk"]), ptr(st["pv"]), ptr(rs), ptr(rp),
+                                               None if one_row else ptr(blk), n_blk, one_row, H, G, d, d, dec.t_max, dec.n_pool_max, SAKINEX_WINDOW,
+                                               SAKINEX_POOL, 1.0, ptr(att), H * d, None, 0, ns, ptr(aws), aws.numel(), current_stream()),
+              "mn_window_pool_attn_blocks")
+        return ns
 
     def keys_at(i):
         return min(i + 1, SAKINEX_WINDOW) + max(0, (i - SAKINEX_WINDOW + 1) // SAKINEX_POOL)
-    t = _time(lambda: attn(T, tabs["row_seq"], tabs["row_slot"]), 5)
+    t = _time(lambda: attn(T, tabs["row_seq"], tabs["row_slot"], 0), 5)
     flops = 2 * 2 * H * d * sum(keys_at(i) for i in range(T))
     out["attn_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / FMA_F32_TFLOPS, peak="fp32 FMA")
     for B in batches:
         row_seq = torch.arange(B, dtype=torch.int32, device=dev)
         slot = torch.full((B,), T - 1, dtype=torch.int32, device=dev)
-        t = _time(lambda: attn(B, row_seq, slot), 20)
+        t = _time(lambda: attn(B, row_seq, slot, 1), 20)
         byts = B * keys_at(T - 1) * G * 2 * d * 4
-        out[f"attn_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS, keys=keys_at(T - 1))
+        out[f"attn_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS, keys=keys_at(T - 1),
+                                        key_splits=attn(B, row_seq, slot, 1))
     # the recurrence alone: reads z, u, g, writes the gated state (fp32 rows)
     n = s["width"]
     zx, gg, o = torch.randn(T, 2 * n, device=dev), torch.randn(T, n, device=dev), torch.empty(T, n, device=dev)
-    t = _time(lambda: check(lib().mn_mingru_rows(ptr(zx), 2 * n, ptr(gg), n, ptr(st["gru"]), ptr(tabs["row_seq"]), ptr(tabs["row_slot"]),
-                                                 ptr(tabs["row_back"]), 1.0, ptr(o), n, None, 0, T, n, current_stream()), "mn_mingru_rows"), 5)
+    gws = torch.empty(lib().mn_mingru_scan_workspace_bytes(T, n), dtype=torch.uint8, device=dev)
+    t = _time(lambda: check(lib().mn_mingru_rows_scan(ptr(zx), 2 * n, ptr(gg), n, ptr(st["gru"]), ptr(tabs["row_seq"]), ptr(tabs["row_slot"]),
+                                                      ptr(tabs["row_back"]), 1.0, ptr(o), n, None, 0, T, n, ptr(gws), gws.numel(), current_stream()),
+                            "mn_mingru_rows_scan"), 5)
     out["mingru_prefill"] = dict(us=t * 1e6, gbs=T * n * 16 / t / 1e9, of_peak=T * n * 16 / t / 1e9 / HBM_GBS)
     return out
 
