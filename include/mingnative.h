@@ -902,6 +902,14 @@ MN_API int mn_rotary_frequencies_host(int dims, double base, double factor, doub
 MN_API int mn_rope_unit_append(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, int rot_dims, const float* freq,
                                float mag, int unit, float eps, float q_scale, const int32_t* row_seq, const int32_t* row_slot, float* q_out,
                                int64_t ldq, float* k_arena, float* v_arena, int t_max, void* stream);
+/* Decode rows (every row alone in its sequence) in one launch: qkv holds the UNFILTERED projections; every channel goes through the
+ * causal filter w_conv bf16 [channels, conv] over the sequence's earlier inputs in conv_state fp32 [n_seq, conv - 1, channels], which
+ * moves on by this row (conv 0: no filter); then mn_rope_unit_append; then, for a row that completes a block of `pool` slots, the
+ * block's mean key / value as mn_pool_blocks_update writes them (pool 0: none). */
+MN_API int mn_filter_rope_append_rows(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, const uint16_t* w_conv, int conv,
+                                      float* conv_state, int rot_dims, const float* freq, float mag, int unit, float eps, float q_scale,
+                                      const int32_t* row_seq, const int32_t* row_slot, float* q_out, int64_t ldq, float* k_arena,
+                                      float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool, void* stream);
 /* Mean key / value of every block of `pool` slots that a row of this call completes (row_slot % pool == pool - 1):
  * pk [n_seq, n_pool_max, G * dim], pv [n_seq, n_pool_max, G * vdim], block b of a sequence = its slots [b pool, (b + 1) pool). */
 MN_API int mn_pool_blocks_update(const float* k_arena, const float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool,

@@ -217,17 +217,23 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
     // ---- mixer sublayer ----
     MN_TRY(norm_stage(l.norm1, l.canon1, st->canon[ri], &h, &h16));
     MN_TRY(linear(arith, M, h, W, h16, W, l.w_in, d.n_in, W, l.b_in, pin, d.n_in, gws, gwb, stream));
-    const float* qkv = pin; int64_t ldqkv = d.n_in;
-    if (l.conv >= 1) {
-      MN_TRY(mn_tap_conv_rows(pin, d.n_in, l.w_conv, l.conv, st->conv[ri], row_seq, row_slot, row_back, qkvc, d.cqkv, M, d.cqkv, stream));
-      MN_TRY(mn_tap_state_update(pin, d.n_in, l.conv, st->conv[ri], row_seq, row_back, M, d.cqkv, stream));
-      qkv = qkvc; ldqkv = d.cqkv;
+    if (one_row) {        // decode rows: channel filter + state, rotation, unit norm, append and block means in one launch
+      MN_TRY(mn_filter_rope_append_rows(pin, d.n_in, M, l.heads, l.kv_heads, l.dim, l.vdim, l.w_conv, l.conv, st->conv[ri], l.rot_dims, l.rot_freq,
+                                        l.rot_mag, l.unit_qk, m->eps, l.scale, row_seq, row_slot, qf, d.cq, st->k[ri], st->v[ri], st->t_max,
+                                        st->pk[ri], st->pv[ri], st->n_pool_max, l.pool, stream));
+    } else {
+      const float* qkv = pin; int64_t ldqkv = d.n_in;
+      if (l.conv >= 1) {
+        MN_TRY(mn_tap_conv_rows(pin, d.n_in, l.w_conv, l.conv, st->conv[ri], row_seq, row_slot, row_back, qkvc, d.cqkv, M, d.cqkv, stream));
+        MN_TRY(mn_tap_state_update(pin, d.n_in, l.conv, st->conv[ri], row_seq, row_back, M, d.cqkv, stream));
+        qkv = qkvc; ldqkv = d.cqkv;
+      }
+      MN_TRY(mn_rope_unit_append(qkv, ldqkv, M, l.heads, l.kv_heads, l.dim, l.vdim, l.rot_dims, l.rot_freq, l.rot_mag, l.unit_qk, m->eps, l.scale,
+                                 row_seq, row_slot, qf, d.cq, st->k[ri], st->v[ri], st->t_max, stream));
+      if (l.pool > 0)
+        MN_TRY(mn_pool_blocks_update(st->k[ri], st->v[ri], st->t_max, st->pk[ri], st->pv[ri], st->n_pool_max, l.pool, d.ck, d.cv, row_seq,
+                                     row_slot, M, stream));
     }
-    MN_TRY(mn_rope_unit_append(qkv, ldqkv, M, l.heads, l.kv_heads, l.dim, l.vdim, l.rot_dims, l.rot_freq, l.rot_mag, l.unit_qk, m->eps, l.scale,
-                               row_seq, row_slot, qf, d.cq, st->k[ri], st->v[ri], st->t_max, stream));
-    if (l.pool > 0)
-      MN_TRY(mn_pool_blocks_update(st->k[ri], st->v[ri], st->t_max, st->pk[ri], st->pv[ri], st->n_pool_max, l.pool, d.ck, d.cv, row_seq,
-                                   row_slot, M, stream));
     {
       const int rb = one_row ? 1 : mn_window_attn_block_rows();
       int max_keys = max_len;

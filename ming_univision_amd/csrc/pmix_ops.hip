@@ -7,6 +7,7 @@
 //   mn_axpy_rms_filter_rows    the same for decode rows, with the sublayer-input filter and its state update in the launch
 //   mn_rope_unit_append        rotary (frequency table) + unit-RMS per head on q and k, q scaled, k / v appended to their arenas
 //   mn_pool_blocks_update      mean key / value of the blocks a step completes
+//   mn_filter_rope_append_rows decode rows: the q / k / v channel filter with its state, the rotation and append, the block means — one launch
 //   mn_window_pool_attn        softmax over the window's tokens and the block means before it, online softmax in fp32
 //   mn_window_pool_attn_blocks the same, tiled: runs of rows and query heads share key tiles, key splits with a merge launch
 //   mn_mingru_rows             S = (1 - z) S + z c over each sequence's rows, gated output (mn_mingru_rows_scan: as a chunked scan)
@@ -91,16 +92,19 @@ __global__ __launch_bounds__(256) void axpy_rms_filter_kernel(AxpyRmsFilterArgs 
   const bool filter = a.taps_w != nullptr && a.taps >= 1;
   const int seq = filter ? a.row_seq[row] : 0, slot = filter ? a.row_slot[row] : 0;
   float* const st0 = (filter && a.taps > 1) ? a.state + (int64_t)seq * (a.taps - 1) * n : nullptr;
-  float xv[VPT], sv[VPT][FUSED_MAX_TAPS - 1];
-  // every load of the row is issued before the first store
+  float xv[VPT], sv[VPT][FUSED_MAX_TAPS - 1], wv[VPT], tv[VPT][FUSED_MAX_TAPS];
+  // every load of the row — inputs, state, norm weight, filter taps — is issued before the reduction, and before the first store
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const int c = tid + 256 * i, cc = c < n ? c : 0;
     float t = a.x[(int64_t)row * a.ldx + cc];
     if (a.y) t += a.mult * a.y[(int64_t)row * a.ldy + cc];
     xv[i] = c < n ? t : 0.f;
+    wv[i] = bf16_to_f32(a.w[cc]);
 #pragma unroll
     for (int k = 1; k < FUSED_MAX_TAPS; ++k) sv[i][k - 1] = (st0 && k < a.taps) ? st0[(int64_t)(k - 1) * n + cc] : 0.f;
+#pragma unroll
+    for (int k = 0; k < FUSED_MAX_TAPS; ++k) tv[i][k] = (filter && k < a.taps) ? bf16_to_f32(a.taps_w[(int64_t)cc * a.taps + (a.taps - 1 - k)]) : 0.f;
   }
   float s = 0.f;
 #pragma unroll
@@ -111,14 +115,13 @@ __global__ __launch_bounds__(256) void axpy_rms_filter_kernel(AxpyRmsFilterArgs 
     const int c = tid + 256 * i;
     if (c >= n) continue;
     if (a.y) a.x[(int64_t)row * a.ldx + c] = xv[i];
-    const float nv = xv[i] * r * bf16_to_f32(a.w[c]);
+    const float nv = xv[i] * r * wv[i];
     float acc = nv;
     if (filter) {
-      const bf16_t* tw = a.taps_w + (int64_t)c * a.taps;
-      acc += bf16_to_f32(tw[a.taps - 1]) * nv;
+      acc += tv[i][0] * nv;                              // tv[k]: the tap on the input k positions back
 #pragma unroll
       for (int k = 1; k < FUSED_MAX_TAPS; ++k)
-        if (k < a.taps && slot - k >= 0) acc += bf16_to_f32(tw[a.taps - 1 - k]) * sv[i][k - 1];
+        if (k < a.taps && slot - k >= 0) acc += tv[i][k] * sv[i][k - 1];
       if (st0) {
         float* st = st0 + c;
 #pragma unroll
@@ -141,27 +144,61 @@ struct RopeArgs {
   const int32_t* row_seq; const int32_t* row_slot;
   float* q_out; int64_t ldq;
   float* k_arena; float* v_arena; int t_max;
+  // decode rows only (ROW): the channel filter in front with its state, and the block means behind
+  const bf16_t* w_conv; int conv; float* conv_state;
+  float* pk; float* pv; int n_pool_max, pool;
 };
 
+// ROW: every row is alone in its sequence (a decode step).  The kernel then reads its channels through the short causal filter
+// (taps from w_conv, the sequence's earlier inputs from conv_state, which it moves on) and, when the row completes a block of
+// `pool` slots, writes the block's mean key / value too: mn_tap_conv_rows + mn_tap_state_update + the rotation + mn_pool_blocks_update
+// of such a row in one launch.  Every channel is read by exactly one lane.
+template <bool ROW>
 __global__ __launch_bounds__(256) void rope_unit_append_kernel(RopeArgs a, int M) {
   const int hv = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, m = blockIdx.y;
   const int nh = a.H + 2 * a.G;
   if (hv >= nh) return;
-  const float* src = a.qkv + (int64_t)m * a.ldqkv;
-  const int64_t crow = (int64_t)a.row_seq[m] * a.t_max + a.row_slot[m];
-  if (hv >= a.H + a.G) {                                         // a value head: copied into its arena
+  const float* row = a.qkv + (int64_t)m * a.ldqkv;
+  const int seq = a.row_seq[m], slot = a.row_slot[m];
+  const int64_t crow = (int64_t)seq * a.t_max + slot;
+  const int C = (a.H + a.G) * a.dim + a.G * a.vdim;
+  const bool do_pool = ROW && a.pool > 0 && (slot % a.pool) == a.pool - 1 && slot / a.pool < a.n_pool_max;
+  auto ld = [&](int ch) -> float {
+    const float cur = row[ch];
+    if (!ROW || a.conv < 1) return cur;
+    const bf16_t* w = a.w_conv + (int64_t)ch * a.conv;
+    float acc = bf16_to_f32(w[a.conv - 1]) * cur;
+    if (a.conv > 1) {
+      float* st = a.conv_state + (int64_t)seq * (a.conv - 1) * C + ch;
+      for (int k = 1; k < a.conv; ++k)
+        if (slot - k >= 0) acc += bf16_to_f32(w[a.conv - 1 - k]) * st[(int64_t)(k - 1) * C];
+      for (int k = a.conv - 2; k >= 1; --k) st[(int64_t)k * C] = st[(int64_t)(k - 1) * C];
+      st[0] = cur;
+    }
+    return acc;
+  };
+  auto put = [&](float* arena, float* parena, int n_ch, int c, float val) {      // append, and the block's mean when this row completes it
+    arena[crow * n_ch + c] = val;
+    if (do_pool) {
+      const int b = slot / a.pool;
+      const float* src = arena + ((int64_t)seq * a.t_max + (int64_t)b * a.pool) * n_ch + c;
+      float s = 0.f;
+      for (int j = 0; j < a.pool - 1; ++j) s += src[(int64_t)j * n_ch];
+      s += val;
+      parena[((int64_t)seq * a.n_pool_max + b) * n_ch + c] = s / (float)a.pool;
+    }
+  };
+  if (hv >= a.H + a.G) {                                         // a value head: into its arena
     const int g = hv - a.H - a.G;
-    src += (int64_t)(a.H + a.G) * a.dim + (int64_t)g * a.vdim;
-    float* dst = a.v_arena + crow * ((int64_t)a.G * a.vdim) + (int64_t)g * a.vdim;
-    for (int i = lane; i < a.vdim; i += 64) dst[i] = src[i];
+    for (int i = lane; i < a.vdim; i += 64) put(a.v_arena, a.pv, a.G * a.vdim, g * a.vdim + i, ld((a.H + a.G) * a.dim + g * a.vdim + i));
     return;
   }
   const bool is_q = hv < a.H;
-  src += (int64_t)hv * a.dim;
-  float* dst = is_q ? a.q_out + (int64_t)m * a.ldq + (int64_t)hv * a.dim
-                    : a.k_arena + crow * ((int64_t)a.G * a.dim) + (int64_t)(hv - a.H) * a.dim;
+  const int ch0 = hv * a.dim;
+  float* qdst = a.q_out + (int64_t)m * a.ldq + (int64_t)hv * a.dim;
+  const int kc0 = (hv - a.H) * a.dim;
   const int half = a.rot_dims / 2;
-  const float pos = (float)a.row_slot[m];
+  const float pos = (float)slot;
   float lo[4], hi[4], rest[8];
   float ss = 0.f;
 #pragma unroll
@@ -169,7 +206,7 @@ __global__ __launch_bounds__(256) void rope_unit_append_kernel(RopeArgs a, int M
     const int i = lane + 64 * j;
     lo[j] = hi[j] = 0.f;
     if (i < half) {
-      const float u = src[i], v = src[i + half];
+      const float u = ld(ch0 + i), v = ld(ch0 + i + half);
       const float ang = pos * a.freq[i];
       const float c = cosf(ang) * a.mag, s = sinf(ang) * a.mag;
       lo[j] = u * c - v * s;
@@ -181,7 +218,7 @@ __global__ __launch_bounds__(256) void rope_unit_append_kernel(RopeArgs a, int M
   for (int j = 0; j < 8; ++j) {
     const int i = a.rot_dims + lane + 64 * j;
     rest[j] = 0.f;
-    if (i < a.dim) { rest[j] = src[i]; ss += rest[j] * rest[j]; }
+    if (i < a.dim) { rest[j] = ld(ch0 + i); ss += rest[j] * rest[j]; }
   }
   float r = 1.0f;
   if (a.unit) r = 1.0f / sqrtf(wave_sum(ss) / (float)a.dim + a.eps);
@@ -189,12 +226,18 @@ __global__ __launch_bounds__(256) void rope_unit_append_kernel(RopeArgs a, int M
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int i = lane + 64 * j;
-    if (i < half) { dst[i] = lo[j] * r; dst[i + half] = hi[j] * r; }
+    if (i < half) {
+      if (is_q) { qdst[i] = lo[j] * r; qdst[i + half] = hi[j] * r; }
+      else { put(a.k_arena, a.pk, a.G * a.dim, kc0 + i, lo[j] * r); put(a.k_arena, a.pk, a.G * a.dim, kc0 + i + half, hi[j] * r); }
+    }
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int i = a.rot_dims + lane + 64 * j;
-    if (i < a.dim) dst[i] = rest[j] * r;
+    if (i < a.dim) {
+      if (is_q) qdst[i] = rest[j] * r;
+      else put(a.k_arena, a.pk, a.G * a.dim, kc0 + i, rest[j] * r);
+    }
   }
 }
 
@@ -784,9 +827,27 @@ extern "C" int mn_rope_unit_append(const float* qkv, int64_t ldqkv, int M, int H
                "mn_rope_unit_append: bad args");
   MN_CHECK_ARG(dim >= 1 && dim <= 512 && vdim >= 1 && rot_dims >= 0 && rot_dims <= dim && (rot_dims % 2) == 0 && (rot_dims == 0 || freq),
                "mn_rope_unit_append: dim=%d (at most 512), rot_dims=%d (even, at most dim)", dim, rot_dims);
-  RopeArgs a{qkv, ldqkv, H, G, dim, vdim, rot_dims, freq, mag, unit, eps, q_scale, row_seq, row_slot, q_out, ldq, k_arena, v_arena, t_max};
-  hipLaunchKernelGGL(rope_unit_append_kernel, dim3((unsigned)mn_cdiv(H + 2 * G, 4), (unsigned)M), dim3(256), 0, mn_stream(stream), a, M);
+  RopeArgs a{qkv, ldqkv, H, G, dim, vdim, rot_dims, freq, mag, unit, eps, q_scale, row_seq, row_slot, q_out, ldq, k_arena, v_arena, t_max,
+             nullptr, 0, nullptr, nullptr, nullptr, 0, 0};
+  hipLaunchKernelGGL((rope_unit_append_kernel<false>), dim3((unsigned)mn_cdiv(H + 2 * G, 4), (unsigned)M), dim3(256), 0, mn_stream(stream), a, M);
   MN_CHECK_LAUNCH("mn_rope_unit_append");
+  return MN_OK;
+}
+
+extern "C" int mn_filter_rope_append_rows(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, const uint16_t* w_conv, int conv,
+                                          float* conv_state, int rot_dims, const float* freq, float mag, int unit, float eps, float q_scale,
+                                          const int32_t* row_seq, const int32_t* row_slot, float* q_out, int64_t ldq, float* k_arena,
+                                          float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool, void* stream) {
+  MN_CHECK_ARG(qkv && row_seq && row_slot && q_out && k_arena && v_arena && M >= 1 && M <= 65535 && H >= 1 && G >= 1 && t_max >= 1,
+               "mn_filter_rope_append_rows: bad args");
+  MN_CHECK_ARG(dim >= 1 && dim <= 512 && vdim >= 1 && rot_dims >= 0 && rot_dims <= dim && (rot_dims % 2) == 0 && (rot_dims == 0 || freq),
+               "mn_filter_rope_append_rows: dim=%d (at most 512), rot_dims=%d (even, at most dim)", dim, rot_dims);
+  MN_CHECK_ARG(conv >= 0 && (conv == 0 || w_conv) && (conv <= 1 || conv_state) && pool >= 0 && (pool == 0 || (pk && pv && n_pool_max >= 1)),
+               "mn_filter_rope_append_rows: bad filter or block arenas");
+  RopeArgs a{qkv, ldqkv, H, G, dim, vdim, rot_dims, freq, mag, unit, eps, q_scale, row_seq, row_slot, q_out, ldq, k_arena, v_arena, t_max,
+             w_conv, conv, conv_state, pk, pv, n_pool_max, pool};
+  hipLaunchKernelGGL((rope_unit_append_kernel<true>), dim3((unsigned)mn_cdiv(H + 2 * G, 4), (unsigned)M), dim3(256), 0, mn_stream(stream), a, M);
+  MN_CHECK_LAUNCH("mn_filter_rope_append_rows");
   return MN_OK;
 }
 

@@ -205,6 +205,48 @@ def test_rotation_unit_norm_and_append(H, G, dim, vdim, rot):
     assert int((ka != 0).any(-1).sum()) == M
 
 
+@pytest.mark.parametrize("H,G,dim,vdim,conv,pool,dims", [(4, 2, 16, 24, 3, 4, 8), (3, 1, 12, 20, 2, 3, 6), (2, 2, 16, 16, 1, 1, 16), (2, 1, 8, 8, 0, 0, 0),
+                                                         (1, 1, 136, 8, 5, 2, 130)])
+def test_decode_rows_filter_rotation_append_and_block_means_in_one_launch(H, G, dim, vdim, conv, pool, dims):
+    """The fused launch of decode rows against the chain of operators it stands for (channel filter, its state update, rotation and
+    append, block means), on rows of four sequences at positions that do and do not complete a block and have less history than taps."""
+    from ming_univision_amd.sakinex import rotary_table
+    check, stream, L, ptr = _api()
+    g = torch.Generator().manual_seed(11)
+    C, t_max, M, n_seq = (H + G) * dim + G * vdim, 40, 4, 5
+    npm = t_max // max(pool, 1) + 1
+    freq, mag = rotary_table(dict(base=50.0, dims=dims, scaling=dict(factor=4.0, fast=8.0, original=16, slow=1.0)), "cuda") if dims else (None, 1.0)
+    pin = torch.randn(M, C + 7, generator=g).cuda()
+    w = _bf(torch.randn(C, max(conv, 1), generator=g)).cuda()
+    seq = torch.tensor([3, 0, 4, 1], dtype=torch.int32).cuda()
+    slot = torch.tensor([0, 1, 2 * max(pool, 1) - 1 + 8, 11], dtype=torch.int32).cuda()
+    back = torch.zeros(M, dtype=torch.int32).cuda()
+    init = dict(state=torch.randn(n_seq, max(conv - 1, 1), C, generator=g), ka=torch.randn(n_seq, t_max, G * dim, generator=g),
+                va=torch.randn(n_seq, t_max, G * vdim, generator=g), pk=torch.randn(n_seq, npm, G * dim, generator=g),
+                pv=torch.randn(n_seq, npm, G * vdim, generator=g))
+    a = {k: v.cuda() for k, v in init.items()}
+    b = {k: v.cuda() for k, v in init.items()}
+    qa, qb, tmp = torch.empty(M, H * dim, device="cuda"), torch.empty(M, H * dim, device="cuda"), torch.empty(M, C, device="cuda")
+    src, ld = pin, C + 7
+    if conv:
+        check(L.mn_tap_conv_rows(ptr(pin), C + 7, ptr(w), conv, ptr(a["state"]), ptr(seq), ptr(slot), ptr(back), ptr(tmp), C, M, C, stream()))
+        check(L.mn_tap_state_update(ptr(pin), C + 7, conv, ptr(a["state"]), ptr(seq), ptr(back), M, C, stream()))
+        src, ld = tmp, C
+    check(L.mn_rope_unit_append(ptr(src), ld, M, H, G, dim, vdim, dims, ptr(freq), mag, 1, 1e-6, 0.3, ptr(seq), ptr(slot), ptr(qa), H * dim, ptr(a["ka"]),
+                                ptr(a["va"]), t_max, stream()))
+    if pool:
+        check(L.mn_pool_blocks_update(ptr(a["ka"]), ptr(a["va"]), t_max, ptr(a["pk"]), ptr(a["pv"]), npm, pool, G * dim, G * vdim, ptr(seq), ptr(slot), M,
+                                      stream()))
+    check(L.mn_filter_rope_append_rows(ptr(pin), C + 7, M, H, G, dim, vdim, ptr(w) if conv else None, conv, ptr(b["state"]), dims, ptr(freq), mag, 1, 1e-6,
+                                       0.3, ptr(seq), ptr(slot), ptr(qb), H * dim, ptr(b["ka"]), ptr(b["va"]), t_max, ptr(b["pk"]) if pool else None,
+                                       ptr(b["pv"]) if pool else None, npm, pool, stream()))
+    assert err(qb, qa.cpu()) < 1e-6
+    for k in a:
+        assert err(b[k], a[k].cpu()) < 1e-6, k
+    assert pool == 0 or not torch.equal(a["pk"].cpu(), init["pk"])          # some row did complete a block
+    assert conv <= 1 or not torch.equal(a["state"].cpu(), init["state"])
+
+
 def _attention_case(T, H, G, dim, vdim, window, pool, peaky, seed, rows=None):
     """Random unit-norm keys in an arena, the block means by the framework's own kernel, attention of `rows` (default all) against
     the oracle's."""
