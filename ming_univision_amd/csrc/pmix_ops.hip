@@ -85,14 +85,20 @@ struct AxpyRmsFilterArgs {
   int n;
 };
 
-template <int VPT>
+// MT: the most taps this instance holds in registers (4 or 8)
+template <int VPT, int MT>
 __global__ __launch_bounds__(256) void axpy_rms_filter_kernel(AxpyRmsFilterArgs a) {
   __shared__ float red[8];
   const int row = blockIdx.x, tid = threadIdx.x, n = a.n;
   const bool filter = a.taps_w != nullptr && a.taps >= 1;
   const int seq = filter ? a.row_seq[row] : 0, slot = filter ? a.row_slot[row] : 0;
   float* const st0 = (filter && a.taps > 1) ? a.state + (int64_t)seq * (a.taps - 1) * n : nullptr;
-  float xv[VPT], sv[VPT][FUSED_MAX_TAPS - 1], wv[VPT], tv[VPT][FUSED_MAX_TAPS];
+  float xv[VPT], sv[VPT][MT - 1], wv[VPT], tv[VPT][MT];
+  const float* sbase = st0 ? st0 : a.x + (int64_t)row * a.ldx;         // without a state: any readable row, stride 0
+  const int64_t sstr = st0 ? n : 0;
+  const int ns = st0 ? a.taps - 1 : 1;                                  // state entries
+  const bf16_t* tbase = filter ? a.taps_w : a.w;                        // without a filter: the norm weight, stride 0
+  const int tstr = filter ? a.taps : 0, nt = filter ? a.taps : 1;
   // every load of the row — inputs, state, norm weight, filter taps — is issued before the reduction, and before the first store
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
@@ -101,10 +107,18 @@ __global__ __launch_bounds__(256) void axpy_rms_filter_kernel(AxpyRmsFilterArgs 
     if (a.y) t += a.mult * a.y[(int64_t)row * a.ldy + cc];
     xv[i] = c < n ? t : 0.f;
     wv[i] = bf16_to_f32(a.w[cc]);
+    // unconditional loads at clamped (always valid) addresses, the unused ones zeroed afterwards: a load under a branch would wait
+    // for its value before the next branch, one round trip per tap
 #pragma unroll
-    for (int k = 1; k < FUSED_MAX_TAPS; ++k) sv[i][k - 1] = (st0 && k < a.taps) ? st0[(int64_t)(k - 1) * n + cc] : 0.f;
+    for (int k = 1; k < MT; ++k) {
+      const float v = sbase[(int64_t)(min(k, ns) - 1) * sstr + cc];
+      sv[i][k - 1] = (st0 && k < a.taps) ? v : 0.f;
+    }
 #pragma unroll
-    for (int k = 0; k < FUSED_MAX_TAPS; ++k) tv[i][k] = (filter && k < a.taps) ? bf16_to_f32(a.taps_w[(int64_t)cc * a.taps + (a.taps - 1 - k)]) : 0.f;
+    for (int k = 0; k < MT; ++k) {
+      const float v = bf16_to_f32(tbase[(int64_t)cc * tstr + max(nt - 1 - k, 0)]);
+      tv[i][k] = (filter && k < a.taps) ? v : 0.f;
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -120,12 +134,12 @@ __global__ __launch_bounds__(256) void axpy_rms_filter_kernel(AxpyRmsFilterArgs 
     if (filter) {
       acc += tv[i][0] * nv;                              // tv[k]: the tap on the input k positions back
 #pragma unroll
-      for (int k = 1; k < FUSED_MAX_TAPS; ++k)
+      for (int k = 1; k < MT; ++k)
         if (k < a.taps && slot - k >= 0) acc += tv[i][k] * sv[i][k - 1];
       if (st0) {
         float* st = st0 + c;
 #pragma unroll
-        for (int k = FUSED_MAX_TAPS - 2; k >= 1; --k)
+        for (int k = MT - 2; k >= 1; --k)
           if (k < a.taps - 1) st[(int64_t)k * n] = sv[i][k - 1];
         st[0] = nv;
       }
@@ -582,17 +596,16 @@ __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
   // the weight of every (vector, split) once per workgroup: exp(its maximum - the overall maximum), and the vectors' normalisers
   __shared__ float wgt[AQ * 64];
   __shared__ float Ls[AQ];
-  if (tid < AQ) {
-    float mx = -INFINITY;
-    for (int s = 0; s < a.nsplit; ++s) mx = fmaxf(mx, base[s * stride + tid]);
-    float L = 0.f;
-    for (int s = 0; s < a.nsplit; ++s) {
-      const float ms = base[s * stride + tid];
-      const float w = ms == -INFINITY ? 0.f : expf(ms - mx);
-      wgt[tid * 64 + s] = w;
-      L = fmaf(base[s * stride + AQ + tid], w, L);
-    }
-    Ls[tid] = L;
+  for (int i = tid >> 6; i < AQ; i += 4) {            // one wave per vector, one lane per split (at most 64)
+    const int lane = tid & 63;
+    const bool on = lane < a.nsplit;
+    const float ms = on ? base[lane * stride + i] : -INFINITY;
+    const float ls = on ? base[lane * stride + AQ + i] : 0.f;
+    const float mx = wave_max(ms);
+    const float w = ms == -INFINITY ? 0.f : expf(ms - mx);
+    wgt[i * 64 + lane] = w;
+    const float L = wave_sum(ls * w);
+    if (lane == 0) Ls[i] = L;
   }
   __syncthreads();
   for (int e = tid; e < nqv * a.vdim; e += 256) {
@@ -812,7 +825,11 @@ extern "C" int mn_axpy_rms_filter_rows(float* x, int64_t ldx, const float* y, in
   AxpyRmsFilterArgs a{x, ldx, y, ldy, mult, w, eps, taps_w, taps_w ? taps : 0, state, row_seq, row_slot, h, ldh, n};
   const int vpt = (n + 255) / 256;
   hipStream_t st = mn_stream(stream);
-#define MN_RB(V_) hipLaunchKernelGGL((axpy_rms_filter_kernel<V_>), dim3((unsigned)M), dim3(256), 0, st, a)
+#define MN_RB(V_)                                                                                                   \
+  do {                                                                                                              \
+    if (a.taps <= 4) hipLaunchKernelGGL((axpy_rms_filter_kernel<V_, 4>), dim3((unsigned)M), dim3(256), 0, st, a); \
+    else hipLaunchKernelGGL((axpy_rms_filter_kernel<V_, 8>), dim3((unsigned)M), dim3(256), 0, st, a);             \
+  } while (0)
   if (vpt <= 1) MN_RB(1); else if (vpt <= 2) MN_RB(2); else if (vpt <= 4) MN_RB(4); else if (vpt <= 8) MN_RB(8);
   else if (vpt <= 16) MN_RB(16); else MN_RB(32);
 #undef MN_RB
