@@ -54,7 +54,7 @@ def pizitar_config(s):
 def sakinex_config(s):
     from .configuration import SakinexConfig
     left = dict(conv=4, dim=128, vdim=128, heads=s["heads"], kv_heads=s["heads"] // 4, mask=dict(pool=SAKINEX_POOL, size=SAKINEX_WINDOW),
-                rot=dict(base=600000.0, dims=128, scaling=dict(factor=8.0, fast=32.0, original=4096, slow=1.0)), scale=128 ** -0.5)
+                rot=dict(base=600000.0, dims=128, scaling=dict(factor=4.0, fast=16.0, original=4096, slow=1.0)), scale=128 ** -0.5)
     ly = dict(type="parallel", mixer=dict(left=left, left_scale=0.7, right=dict(width=s["width"]), right_scale=0.7),
               mlp=dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=s["ff"] // 2), shared=dict(ff=s["ff"] // 2)))
     return SakinexConfig(width=s["width"], vocab=s["vocab"], layers=[ly] * s["layers"], canon=dict(taps=4), norm=dict(eps=1e-6), residual_mult=0.5)

@@ -33,7 +33,7 @@ def test_config_and_registry(tmp_path):
 
 
 @pytest.mark.parametrize("loop,want", [
-    (None, [0, 1, 2, 3]), ((0, 2, 3), [0, 1, 0, 1, 0, 1, 2, 3]), ((1, 2, 2), [0, 1, 1, 2, 3]), ((2, 4, 2), [0, 1, 2, 3, 2, 3]),
+    (None, [0, 1, 2, 3]), ((0, 3, 2), [0, 1, 2, 0, 1, 2, 3]), ((1, 2, 2), [0, 1, 1, 2, 3]), ((2, 4, 2), [0, 1, 2, 3, 2, 3]),
     ((0, 4, 1), [0, 1, 2, 3]), ((3, 3, 5), [0, 1, 2, 3])])
 def test_order_of_layer_runs(loop, want):
     cfg = O.small_config(n_layers=4, loop=loop)
