@@ -936,6 +936,15 @@ MN_API int mn_window_pool_attn_blocks(const float* q, int64_t ldq, const float* 
                                       int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
                                       float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
                                       size_t workspace_bytes, void* stream);
+/* The same with the kernel named: MN_WINDOW_ATTN_MFMA (what mn_window_pool_attn_blocks runs for runs of rows with dim, vdim <= 256) =
+ * scores and weighted sums on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: fp32 operands and accumulation), 16-key tiles with
+ * keys and values staged in LDS; MN_WINDOW_ATTN_VALU = the fp32 FMA kernel (decode rows, larger heads). */
+enum { MN_WINDOW_ATTN_MFMA = 0, MN_WINDOW_ATTN_VALU = 1 };
+MN_API int mn_window_pool_attn_blocks_ex(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk,
+                                         const float* pv, const int32_t* row_seq, const int32_t* row_slot, const int32_t* blk_tab, int n_blk,
+                                         int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
+                                         float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
+                                         size_t workspace_bytes, int variant, void* stream);
 /* minGRU over each sequence's rows: z = sigmoid(zx[m, c]), u = zx[m, n + c] (biases already added), candidate = u + 1/2 (u >= 0) or
  * sigmoid(u); S = (1 - z) S + z candidate from state fp32 [n_seq, n] (a row at slot 0 starts from zero), which is left at the
  * sequence's last row; out[m, c] = out_scale * S * silu(g[m, c]).  Rows of one sequence are consecutive (row_back as in 9). */

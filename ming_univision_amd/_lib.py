@@ -332,6 +332,8 @@ SYMBOLS = {
     "mn_window_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "mn_window_pool_attn_blocks": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64, _i,
                                         _p, _sz, _p]),
+    "mn_window_pool_attn_blocks_ex": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64,
+                                           _i, _p, _sz, _i, _p]),
     "mn_semdec_step": (_i, [C.POINTER(SemDec), _p, _i, _p, _p, _p, _p, _i, _i64, _p, _p, _p, _sz, _p]),
 }
 

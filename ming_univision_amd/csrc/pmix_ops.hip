@@ -18,6 +18,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "mfma_f32_tiles.h"
 
 extern "C" int mn_rotary_frequencies_host(int dims, double base, double factor, double original, double fast, double slow, float* freq,
                                           float* mag) {
@@ -581,6 +582,149 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
   }
 }
 
+// Attention on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: scores and weights stay 32-bit), for runs of rows.  A workgroup of
+// 4 waves owns the same 16 query vectors as the tiled form (<= 4 rows x <= 4 heads of one key/value head) and walks its keys —
+// block means, then tokens — in tiles of 16, keys AND values staged through registers into LDS while the previous tile is multiplied:
+//   scores   S[16 q, 16 keys] = Q K^T: every wave multiplies its quarter of the head's values (its slice of Q stays in registers),
+//            the partial tiles are summed through LDS, so all four waves hold the same scores, apply the same per-(row, key)
+//            visibility and keep the same running maximum / sum
+//   values   O[16 q, vdim] += P V: the weights go through LDS into the A-operand layout, wave w owns the 16-column blocks w, w + 4, ..
+// NBD / NBV: 64-value blocks of a key / a value (zero padded).  Key splits write the same partial layout as the tiled form.
+template <int NBD, int NBV>
+__global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
+  constexpr int KT = 16, LDP = 20, LDS_S = 17, DP = 64 * NBD, VP = 64 * NBV, LDK = DP + 4, LDV = VP + 4, DQ = DP / 4, AQ = 16;
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, b = blockIdx.x, gy = blockIdx.y, sp = blockIdx.z;
+  const int rep = a.H / a.G, chunks = (rep + a.hpc - 1) / a.hpc;
+  const int g = gy / chunks, h0 = g * rep + (gy % chunks) * a.hpc;
+  const int Rc = min(a.hpc, g * rep + rep - h0);
+  const int r0 = a.blk_tab[2 * b];
+  const int nr = min(a.blk_tab[2 * b + 1], a.rows_per_blk);
+  const int nqv = nr * Rc;
+  const int seq = a.row_seq[r0], pos0 = a.row_slot[r0], posL = pos0 + nr - 1;
+  const int nbL = win_nb(posL, a.window, a.pool), tF = win_t0(pos0, a.window);
+  const int nk = nbL + (posL - tF + 1);
+  const int ntile = (nk + KT - 1) / KT, tps = (ntile + a.nsplit - 1) / a.nsplit;
+  const int t0 = sp * tps, t1 = min(ntile, t0 + tps);
+  float* Kl = lds;                       // [16 keys][LDK]
+  float* Vl = Kl + KT * LDK;             // [16 keys][LDV]
+  float* Sp = Vl + KT * LDV;             // [4 waves][16 q][LDS_S] partial scores
+  float* Pl = Sp + 4 * 16 * LDS_S;       // [16 q][LDP] weights
+  const int wave = tid >> 6, lane = tid & 63, c16 = lane & 15, g4 = lane >> 4;
+  // the A operands of this wave's score products stay in registers for the whole key walk: query c16, values wave DQ + 4 it + g4
+  float qreg[DQ / 4];
+  {
+    const int qv = min(c16, nqv - 1);
+    const float* src = a.q + (int64_t)(r0 + qv / Rc) * a.ldq + (int64_t)(h0 + qv % Rc) * a.dim;
+#pragma unroll
+    for (int it = 0; it < DQ / 4; ++it) {
+      const int d = wave * DQ + 4 * it + g4;
+      const float t = src[d < a.dim ? d : 0];
+      qreg[it] = (c16 < nqv && d < a.dim) ? t : 0.f;
+    }
+  }
+  int mypos[4], my_nb[4], my_t0[4];
+  float mrun[4], lrun[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int qv = 4 * g4 + i;
+    mypos[i] = qv < nqv ? pos0 + qv / Rc : -1;              // -1: no such vector, it sees nothing
+    my_nb[i] = qv < nqv ? win_nb(mypos[i], a.window, a.pool) : 0;
+    my_t0[i] = qv < nqv ? win_t0(mypos[i], a.window) : 0;
+    mrun[i] = -INFINITY;
+    lrun[i] = 0.f;
+  }
+  f32x4 acc[NBV];
+#pragma unroll
+  for (int c = 0; c < NBV; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int Gd = a.G * a.dim, Gv = a.G * a.vdim;
+  const float* kb = a.k + ((int64_t)seq * a.t_max + tF) * Gd + (int64_t)g * a.dim;
+  const float* vb = a.v + ((int64_t)seq * a.t_max + tF) * Gv + (int64_t)g * a.vdim;
+  const float* pkb = a.pk ? a.pk + (int64_t)seq * a.n_pool_max * Gd + (int64_t)g * a.dim : nullptr;
+  const float* pvb = a.pv ? a.pv + (int64_t)seq * a.n_pool_max * Gv + (int64_t)g * a.vdim : nullptr;
+  f32x4 vk[NBD], vv[NBV];
+  auto fetch = [&](int tile) {
+    const int k0 = tile * KT;
+    load16<NBD>(vk, a.dim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pkb + (int64_t)jj * Gd : kb + (int64_t)(jj - nbL) * Gd; },
+                [&](int j) { return k0 + j < nk; });
+    load16<NBV>(vv, a.vdim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pvb + (int64_t)jj * Gv : vb + (int64_t)(jj - nbL) * Gv; },
+                [&](int j) { return k0 + j < nk; });
+  };
+  if (t0 < t1) fetch(t0);
+  for (int tile = t0; tile < t1; ++tile) {
+    const int key0 = tile * KT;
+    lds_barrier();                                             // the previous tile's keys, values and weights are consumed
+    store16<NBD, LDK>(Kl, vk, tid);
+    store16<NBV, LDV>(Vl, vv, tid);
+    if (tile + 1 < t1) fetch(tile + 1);                          // in flight while this tile is multiplied
+    lds_barrier();
+    {                                                            // partial scores over this wave's quarter of the head's values
+      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f}, s2 = f32x4{0.f, 0.f, 0.f, 0.f};
+      const float* cb = Kl + c16 * LDK + wave * DQ + g4;
+#pragma unroll
+      for (int it = 0; it < DQ / 4; it += 2) {
+        s = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[it], cb[4 * it], s, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_16x16x4f32(qreg[it + 1], cb[4 * it + 4], s2, 0, 0, 0);
+      }
+      s += s2;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) Sp[(wave * 16 + 4 * g4 + i) * LDS_S + c16] = s[i];
+    }
+    lds_barrier();
+    float corr[4];
+    const int j = key0 + c16, tok = tF + (j - nbL);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int o = (4 * g4 + i) * LDS_S + c16;
+      float sc = (Sp[o] + Sp[16 * LDS_S + o]) + (Sp[32 * LDS_S + o] + Sp[48 * LDS_S + o]);
+      const bool see = j < nk && (j < nbL ? j < my_nb[i] : (tok >= my_t0[i] && tok <= mypos[i]));
+      if (!see) sc = -INFINITY;
+      const float mnew = fmaxf(mrun[i], row16_max(sc));
+      const float p = (sc == -INFINITY) ? 0.f : fast_exp(sc - mnew);
+      corr[i] = (mrun[i] == -INFINITY) ? 0.f : fast_exp(mrun[i] - mnew);
+      lrun[i] = lrun[i] * corr[i] + row16_sum(p);
+      mrun[i] = mnew;
+      if (wave == 0) Pl[(4 * g4 + i) * LDP + c16] = p;
+    }
+#pragma unroll
+    for (int c = 0; c < NBV; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[c][i] *= corr[i];
+    lds_barrier();
+    // step t multiplies keys t, t + 4, t + 8, t + 12 (lane group g4 holds key t + 4 g4): with the row stride 4 mod 32 their rows
+    // start 16 banks apart pairwise
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float pa = Pl[c16 * LDP + t + 4 * g4];
+      const float* cb = Vl + (t + 4 * g4) * LDV + 16 * wave + c16;
+#pragma unroll
+      for (int c = 0; c < NBV; ++c) acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa, cb[64 * c], acc[c], 0, 0, 0);
+    }
+  }
+  float* part_out = a.nsplit > 1 ? a.part + (((int64_t)b * gridDim.y + gy) * a.nsplit + sp) * ((int64_t)AQ * (2 + a.vdim)) : nullptr;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int qv = 4 * g4 + i;
+    if (qv >= nqv) continue;
+    const int row = r0 + qv / Rc;
+    const int64_t col0 = (int64_t)(h0 + qv % Rc) * a.vdim;
+    const float inv = a.out_scale / lrun[i];
+#pragma unroll
+    for (int c = 0; c < NBV; ++c) {
+      const int d = 16 * (wave + 4 * c) + c16;
+      if (d >= a.vdim) continue;
+      if (part_out) {
+        part_out[2 * AQ + (int64_t)qv * a.vdim + d] = acc[c][i];
+      } else {
+        const float val = acc[c][i] * inv;
+        if (a.out) a.out[(int64_t)row * a.ldo + col0 + d] = val;
+        if (a.out16) a.out16[(int64_t)row * a.ldo16 + col0 + d] = f32_to_bf16(val);
+      }
+    }
+    if (part_out && wave == 0 && c16 == 0) { part_out[qv] = mrun[i]; part_out[AQ + qv] = lrun[i]; }
+  }
+}
+
 // grid (n_blk, G * chunks): the splits' statistics and sums of every vector become its result
 template <int AQ>
 __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
@@ -932,6 +1076,18 @@ extern "C" int mn_window_pool_attn_blocks(const float* q, int64_t ldq, const flo
                                           int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
                                           float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
                                           size_t workspace_bytes, void* stream) {
+  // runs of rows with heads of at most 256 values go to the matrix cores, decode rows and larger heads to the fp32 FMA kernel
+  const int variant = (!one_row && dim <= 256 && vdim <= 256) ? MN_WINDOW_ATTN_MFMA : MN_WINDOW_ATTN_VALU;
+  return mn_window_pool_attn_blocks_ex(q, ldq, k_arena, v_arena, pk, pv, row_seq, row_slot, blk_tab, n_blk, one_row, H, G, dim, vdim, t_max,
+                                       n_pool_max, window, pool, out_scale, out, ldo, out16, ldo16, nsplit, workspace, workspace_bytes, variant,
+                                       stream);
+}
+
+extern "C" int mn_window_pool_attn_blocks_ex(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk,
+                                             const float* pv, const int32_t* row_seq, const int32_t* row_slot, const int32_t* blk_tab, int n_blk,
+                                             int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
+                                             float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
+                                             size_t workspace_bytes, int variant, void* stream) {
   MN_CHECK_ARG(q && k_arena && v_arena && row_seq && row_slot && (out || out16) && n_blk >= 1 && H >= 1 && G >= 1 && (H % G) == 0 && dim >= 1 &&
                    vdim >= 1 && vdim <= 512 && t_max >= 1 && window >= 0 && pool >= 0 && nsplit >= 1 && nsplit <= 64,
                "mn_window_pool_attn_blocks: bad args (vdim=%d: at most 512; nsplit=%d: at most 64)", vdim, nsplit);
@@ -941,10 +1097,29 @@ extern "C" int mn_window_pool_attn_blocks(const float* q, int64_t ldq, const flo
   MN_CHECK_ARG((int64_t)G * sh.chunks <= 65535, "mn_window_pool_attn_blocks: too many heads");
   MN_CHECK_ARG(nsplit == 1 || (workspace && workspace_bytes >= mn_window_attn_workspace_bytes(n_blk, H, G, vdim, one_row, nsplit)),
                "mn_window_pool_attn_blocks: workspace too small");
-  const size_t lds = ((size_t)sh.aq * dim + 2 * (size_t)sh.aq * AKT + 3 * sh.aq + (size_t)sh.aq * 256) * sizeof(float);
-  MN_CHECK_ARG(lds <= 64 * 1024, "mn_window_pool_attn_blocks: dim=%d too large", dim);
   AttnTArgs a{q, ldq, k_arena, v_arena, pool ? pk : nullptr, pool ? pv : nullptr, row_seq, row_slot, one_row ? nullptr : blk_tab, H, G, dim, vdim,
               t_max, n_pool_max, window, pool, sh.rows, sh.hpc, nsplit, out_scale, out, ldo, out16, ldo16, (float*)workspace};
+  MN_CHECK_ARG(variant == MN_WINDOW_ATTN_VALU || (variant == MN_WINDOW_ATTN_MFMA && !one_row && dim <= 256 && vdim <= 256),
+               "mn_window_pool_attn_blocks: the matrix-core kernel takes runs of rows with dim, vdim <= 256");
+  if (variant == MN_WINDOW_ATTN_MFMA) {
+    const int nbd = dim <= 64 ? 1 : (dim <= 128 ? 2 : 4), nbv = vdim <= 64 ? 1 : (vdim <= 128 ? 2 : 4);
+    const size_t ldsm = ((size_t)16 * (64 * nbd + 4) + (size_t)16 * (64 * nbv + 4) + 4 * 16 * 17 + 16 * 20) * sizeof(float);
+    const dim3 gridm((unsigned)n_blk, (unsigned)(G * sh.chunks), (unsigned)nsplit);
+    hipStream_t stm = mn_stream(stream);
+#define MN_WM(D_, V_) hipLaunchKernelGGL((window_attn_mfma_kernel<D_, V_>), gridm, dim3(256), ldsm, stm, a)
+    if (nbd == 1) { if (nbv == 1) MN_WM(1, 1); else if (nbv == 2) MN_WM(1, 2); else MN_WM(1, 4); }
+    else if (nbd == 2) { if (nbv == 1) MN_WM(2, 1); else if (nbv == 2) MN_WM(2, 2); else MN_WM(2, 4); }
+    else { if (nbv == 1) MN_WM(4, 1); else if (nbv == 2) MN_WM(4, 2); else MN_WM(4, 4); }
+#undef MN_WM
+    MN_CHECK_LAUNCH("mn_window_pool_attn_blocks(mfma)");
+    if (nsplit > 1) {
+      hipLaunchKernelGGL((window_attn_merge_kernel<16>), dim3((unsigned)n_blk, (unsigned)(G * sh.chunks)), dim3(256), 0, stm, a);
+      MN_CHECK_LAUNCH("mn_window_pool_attn_blocks(merge)");
+    }
+    return MN_OK;
+  }
+  const size_t lds = ((size_t)sh.aq * dim + 2 * (size_t)sh.aq * AKT + 3 * sh.aq + (size_t)sh.aq * 256) * sizeof(float);
+  MN_CHECK_ARG(lds <= 64 * 1024, "mn_window_pool_attn_blocks: dim=%d too large", dim);
   const bool vec = (dim % 4) == 0 && (ldq % 4) == 0 && (((uintptr_t)q | (uintptr_t)k_arena | (uintptr_t)pk) & 15) == 0;
   const dim3 grid((unsigned)n_blk, (unsigned)(G * sh.chunks), (unsigned)nsplit);
   hipStream_t st = mn_stream(stream);

@@ -292,13 +292,18 @@ def _attention_case(T, H, G, dim, vdim, window, pool, peaky, seed, rows=None):
             spans = [(1, past, 0), (1, T - past, past)] if past else [(1, T, 0)]
             tb = rows_of_spans(spans, RB)
             blk = torch.from_numpy(tb["blk_tab"]).cuda()
-            for nsplit in (1, 2):
+            for nsplit, variant in ((1, 0), (2, 0), (5, 0), (1, 1), (2, 1)):          # 0: fp32 matrix cores, 1: fp32 FMA
+                if variant == 0 and max(dim, vdim) > 256:
+                    continue
                 outb = torch.full((T, H * vdim), float("nan"), device="cuda")
+                ob16 = torch.empty(T, H * vdim, dtype=torch.bfloat16, device="cuda")
                 ws = torch.empty(max(16, L.mn_window_attn_workspace_bytes(blk.shape[0], H, G, vdim, 0, nsplit)), dtype=torch.uint8, device="cuda")
-                check(L.mn_window_pool_attn_blocks(ptr(qd), H * dim, ptr(ka), ptr(va), ptr(pk) if pool else None, ptr(pv) if pool else None,
-                                                   ptr(r["row_seq"]), ptr(r["row_slot"]), ptr(blk), blk.shape[0], 0, H, G, dim, vdim, t_max, npm, window,
-                                                   pool, 0.6, ptr(outb), H * vdim, None, 0, nsplit, ptr(ws), ws.numel(), stream()))
-                assert err(outb, 0.6 * ref) < 2e-5, (past, nsplit)
+                check(L.mn_window_pool_attn_blocks_ex(ptr(qd), H * dim, ptr(ka), ptr(va), ptr(pk) if pool else None, ptr(pv) if pool else None,
+                                                      ptr(r["row_seq"]), ptr(r["row_slot"]), ptr(blk), blk.shape[0], 0, H, G, dim, vdim, t_max, npm,
+                                                      window, pool, 0.6, ptr(outb), H * vdim, ptr(ob16), H * vdim, nsplit, ptr(ws), ws.numel(), variant,
+                                                      stream()))
+                assert err(outb, 0.6 * ref) < 2e-5, (past, nsplit, variant)
+                assert err(ob16.float(), 0.6 * ref) < 1e-2
 
 
 @pytest.mark.parametrize("H,G,dim,vdim,window,pool", [(4, 2, 16, 24, 9, 4), (3, 1, 12, 20, 7, 3), (2, 2, 16, 16, 1, 1), (12, 1, 8, 8, 0, 0),
@@ -314,6 +319,8 @@ def test_attention_over_several_key_tiles():
     """More than 256 visible keys: block means and window tokens on both sides of a tile's edge; a window cut by the sequence's start."""
     _attention_case(900, 2, 1, 16, 16, 300, 2, peaky=30.0, seed=5, rows=[0, 1, 254, 255, 256, 257, 299, 300, 301, 511, 512, 513, 555, 811, 812, 899])
     _attention_case(600, 3, 1, 8, 8, 0, 0, peaky=30.0, seed=6, rows=[0, 255, 256, 257, 511, 512, 599])
+    _attention_case(200, 8, 2, 72, 136, 37, 5, peaky=30.0, seed=7)       # every row, in runs: heads of 72 / 136 values (padded 64-blocks)
+    _attention_case(150, 2, 2, 200, 40, 0, 0, peaky=20.0, seed=8)        # one query head per key/value head, no window
 
 
 def test_min_gru_rows_carry_their_state():
