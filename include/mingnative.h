@@ -985,7 +985,7 @@ typedef struct mn_pmix_layer {
   const uint16_t *w_in, *b_in;                     /* [q ; k ; v ; z ; x ; g] rows, bias (zero outside z and x) */
   const uint16_t *w_conv;                          /* [(heads + kv_heads) * dim + kv_heads * vdim, conv] */
   const uint16_t *w_out;                           /* [width, heads * vdim + gru] = [left o | right o] */
-  const uint16_t *w_ff_in, *b_ff_in;               /* [shared gate ; shared up ; router ; shared gate logit] rows, bias (router's) */
+  const uint16_t *w_ff_in, *b_ff_in;               /* [shared gate ; shared up ; router ; shared gate logit ; zero rows up to a multiple of 8], bias (router's) */
   const uint16_t *w_shared_down;                   /* [width, shared_ff] */
   const uint16_t *w_gate_up;                       /* [experts, 2 ff, width] */
   const uint16_t *w_down;                          /* [experts, width, ff] */

@@ -24,7 +24,7 @@ PDims pdims(const mn_pmix_layer& l) {
   d.cqkv = d.cq + d.ck + d.cv;
   d.n_in = d.cqkv + 3 * l.gru;
   d.n_cat = l.heads * l.vdim + l.gru;
-  d.n_ff_in = l.experts > 0 ? 2 * l.shared_ff + l.experts + (l.shared_ff > 0 ? 1 : 0) : 0;
+  d.n_ff_in = l.experts > 0 ? (2 * l.shared_ff + l.experts + (l.shared_ff > 0 ? 1 : 0) + 7) / 8 * 8 : 0;    // zero rows pad the stack to a multiple of 8
   return d;
 }
 

@@ -103,8 +103,9 @@ class SakinexDecoder(SeqDecoder):
                 if taps:
                     L.canon2 = self._p(sd[p + "canon2"])
                 shared = [sd[q + "shared.gate"], sd[q + "shared.up"]] if fs else []
-                L.w_ff_in = self._p(torch.cat(shared + [sd[q + "router"]] + ([sd[q + "shared.sg"]] if fs else []), 0))
-                L.b_ff_in = self._p(torch.cat([torch.zeros(2 * fs, **bf), sd[q + "router.b"], torch.zeros(1 if fs else 0, **bf)]))
+                pad = -(2 * fs + E + (1 if fs else 0)) % 8           # zero rows: the stack's row count a multiple of 8 (the wide GEMM's shapes)
+                L.w_ff_in = self._p(torch.cat(shared + [sd[q + "router"]] + ([sd[q + "shared.sg"]] if fs else []) + [torch.zeros(pad, W, **bf)], 0))
+                L.b_ff_in = self._p(torch.cat([torch.zeros(2 * fs, **bf), sd[q + "router.b"], torch.zeros((1 if fs else 0) + pad, **bf)]))
                 if fs:
                     L.w_shared_down = self._p(sd[q + "shared.down"])
                 L.w_gate_up = self._p(torch.stack([torch.cat([sd[f"{q}e{j}.gate"], sd[f"{q}e{j}.up"]], 0) for j in range(E)]))
