@@ -35,6 +35,8 @@ MODELS = {
                  top=1, ff=32, shared_ff=32, taps=1, loop=(0, 2, 1), mult=1.0),
     # twelve query heads on one key/value head (two chunks of the attention launch), a window longer than any test sequence, more
     # experts than the sorted route takes, the repeated range at the start
+    # layers that differ from each other in every size (edited in config()), a repeated range of two layers at the end
+    "varied": dict(width=72, vocab=50, n_layers=4, loop=(2, 4, 2), no_mlp=(3,)),
     "wide": dict(width=32, vocab=40, n_layers=2, heads=12, kv_heads=1, dim=8, vdim=8, rot_dims=4, window=500, pool=16, gru=24, experts=130,
                  top=4, ff=8, shared_ff=8, loop=(0, 1, 3)),
 }
@@ -42,6 +44,17 @@ MODELS = {
 
 def config(name):
     cfg = O.small_config(**MODELS[name])
+    if name == "varied":                                 # no two layers alike: every size, window, filter and router differs
+        cfg = copy.deepcopy(cfg)
+        a, b = cfg["layers"][1], cfg["layers"][2]
+        a["mixer"]["left"].update(heads=2, kv_heads=1, dim=24, vdim=8, conv=2, scale=0.2, mask={"size": 5, "pool": 2},
+                                  rot={"base": 1000.0, "dims": 24})
+        a["mixer"].update(left_scale=1.1, right_scale=0.3, right={"width": 24})
+        a["mlp"].update(router={"experts": 3, "top": 1}, expert={"ff": 40}, shared={"ff": 72})
+        b["mixer"]["left"].update(heads=6, kv_heads=6, dim=8, vdim=40, conv=5, mask={"size": 33})
+        b["mixer"].update(right={"width": 100})
+        b["mlp"].update(router={"experts": 9, "top": 4}, expert={"ff": 16})
+        b["mlp"].pop("shared")
     if name == "wide":                                   # optional keys left out: no filters, no window, no rotation, no shared expert
         cfg = copy.deepcopy(cfg)
         ly = cfg["layers"][1]
@@ -535,7 +548,7 @@ def test_bf16_arithmetic():
     """Serving arithmetic: portions above 64 rows take the bf16 MFMA products and the experts sorted on the grouped MFMA GEMM (rows
     within 3e-2 of the logits' scale against the oracle, but for at most 8 in 100 whose routing was a close call (130 experts make many); median below 1e-2),
     portions of 9 .. 64 rows the weight-streaming MFMA route on hi/lo rows, rows fed a few at a time fp32 FMA."""
-    for name in ("mixed", "odd", "wide"):                 # "odd": no K is a multiple of 8, "wide": too many experts for the sorted route
+    for name in ("mixed", "odd", "wide", "varied"):       # "odd": no K is a multiple of 8, "wide": too many experts for the sorted route
         cfg, sd, dec = make(name, arith="bf16")
         t = toks(cfg, 100)
         ref = O.forward(cfg, sd, t)
