@@ -905,11 +905,14 @@ MN_API int mn_rope_unit_append(const float* qkv, int64_t ldqkv, int M, int H, in
 /* Decode rows (every row alone in its sequence) in one launch: qkv holds the UNFILTERED projections; every channel goes through the
  * causal filter w_conv bf16 [channels, conv] over the sequence's earlier inputs in conv_state fp32 [n_seq, conv - 1, channels], which
  * moves on by this row (conv 0: no filter); then mn_rope_unit_append; then, for a row that completes a block of `pool` slots, the
- * block's mean key / value as mn_pool_blocks_update writes them (pool 0: none). */
+ * block's mean key / value as mn_pool_blocks_update writes them (pool 0: none).  With gru_n > 0 extra workgroups of the launch run
+ * mn_mingru_rows on the same rows (zx, g, gru_state, gru_scale = its out_scale, gru_out fp32 with row stride ldgo). */
 MN_API int mn_filter_rope_append_rows(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, const uint16_t* w_conv, int conv,
                                       float* conv_state, int rot_dims, const float* freq, float mag, int unit, float eps, float q_scale,
                                       const int32_t* row_seq, const int32_t* row_slot, float* q_out, int64_t ldq, float* k_arena,
-                                      float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool, void* stream);
+                                      float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool, const float* zx,
+                                      int64_t ldzx, const float* g, int64_t ldg, float* gru_state, int gru_n, float gru_scale, float* gru_out,
+                                      int64_t ldgo, void* stream);
 /* Mean key / value of every block of `pool` slots that a row of this call completes (row_slot % pool == pool - 1):
  * pk [n_seq, n_pool_max, G * dim], pv [n_seq, n_pool_max, G * vdim], block b of a sequence = its slots [b pool, (b + 1) pool). */
 MN_API int mn_pool_blocks_update(const float* k_arena, const float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool,
@@ -959,6 +962,10 @@ MN_API int mn_mingru_rows_scan(const float* zx, int64_t ldzx, const float* g, in
                                int64_t ldo16, int M, int n, void* workspace, size_t workspace_bytes, void* stream);
 /* The `top` largest of logits[m, 0 .. E) (ties: the lower index) and the softmax over those alone: idx int32 [M, top], w fp32 [M, top] */
 MN_API int mn_router_topk_rows(const float* logits, int64_t ld, int M, int E, int top, int32_t* idx, float* w, void* stream);
+/* mn_router_topk_rows and y[m, c] = silu(x[m, c]) * x[m, n + c] (fp32) in one launch: the router's pick and the shared expert's
+ * activation of decode rows read the same stacked projection */
+MN_API int mn_router_topk_silu_rows(const float* logits, int64_t ld, int M, int E, int top, int32_t* idx, float* w, const float* x,
+                                    int64_t ldx, float* y, int64_t ldy, int n, void* stream);
 /* y[m, c] = silu(x[m, c]) * x[m, n + c]; y16: optional bf16 copy */
 MN_API int mn_silu_mul_rows(const float* x, int64_t ldx, float* y, int64_t ldy, uint16_t* y16, int64_t ldy16, int M, int n, void* stream);
 /* C[z] fp32 [N] = A[z / a_div] . W[w_idx[z]]^T for z < Z: one input row against the weight block its index names (fp32 FMA; A row

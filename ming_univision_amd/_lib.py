@@ -315,7 +315,8 @@ SYMBOLS = {
                                         C.POINTER(C.c_float)]),
     "mn_rope_unit_append": (_i, [_p, _i64, _i, _i, _i, _i, _i, _i, _p, _f, _i, _f, _f, _p, _p, _p, _i64, _p, _p, _i, _p]),
     "mn_filter_rope_append_rows": (_i, [_p, _i64, _i, _i, _i, _i, _i, _p, _i, _p, _i, _p, _f, _i, _f, _f, _p, _p, _p, _i64, _p, _p, _i, _p, _p, _i,
-                                        _i, _p]),
+                                        _i, _p, _i64, _p, _i64, _p, _i, _f, _p, _i64, _p]),
+    "mn_router_topk_silu_rows": (_i, [_p, _i64, _i, _i, _i, _p, _p, _p, _i64, _p, _i64, _i, _p]),
     "mn_pool_blocks_update": (_i, [_p, _p, _i, _p, _p, _i, _i, _i, _i, _p, _p, _i, _p]),
     "mn_window_pool_attn": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64, _p]),
     "mn_mingru_rows": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _f, _p, _i64, _p, _i64, _i, _i, _p]),

@@ -217,10 +217,12 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
     // ---- mixer sublayer ----
     MN_TRY(norm_stage(l.norm1, l.canon1, st->canon[ri], &h, &h16));
     MN_TRY(linear(arith, M, h, W, h16, W, l.w_in, d.n_in, W, l.b_in, pin, d.n_in, gws, gwb, stream));
+    const bool gru_in_rows = one_row && !cath;      // decode rows without bf16 copies: the recurrence rides the launch below
     if (one_row) {        // decode rows: channel filter + state, rotation, unit norm, append and block means in one launch
       MN_TRY(mn_filter_rope_append_rows(pin, d.n_in, M, l.heads, l.kv_heads, l.dim, l.vdim, l.w_conv, l.conv, st->conv[ri], l.rot_dims, l.rot_freq,
                                         l.rot_mag, l.unit_qk, m->eps, l.scale, row_seq, row_slot, qf, d.cq, st->k[ri], st->v[ri], st->t_max,
-                                        st->pk[ri], st->pv[ri], st->n_pool_max, l.pool, stream));
+                                        st->pk[ri], st->pv[ri], st->n_pool_max, l.pool, pin + d.cqkv, d.n_in, pin + d.cqkv + 2 * l.gru, d.n_in,
+                                        st->gru[ri], gru_in_rows ? l.gru : 0, l.right_scale, cat + l.heads * l.vdim, d.n_cat, stream));
     } else {
       const float* qkv = pin; int64_t ldqkv = d.n_in;
       if (l.conv >= 1) {
@@ -248,7 +250,9 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
                                         d.n_cat, cath, d.n_cat, ns, aws, p.attn_ws, stream));
     }
     const int hv = l.heads * l.vdim;
-    if (M >= 2 * 32 && !one_row)                     // many rows: the recurrence as a chunked scan instead of one thread per channel walking them all
+    if (gru_in_rows) {
+      // done with the filter / rotation launch above
+    } else if (M >= 2 * 32 && !one_row)                     // many rows: the recurrence as a chunked scan instead of one thread per channel walking them all
       MN_TRY(mn_mingru_rows_scan(pin + d.cqkv, d.n_in, pin + d.cqkv + 2 * l.gru, d.n_in, st->gru[ri], row_seq, row_slot, row_back, l.right_scale,
                                  cat + hv, d.n_cat, cath ? cath + hv : nullptr, d.n_cat, M, l.gru, gruws, p.gru_ws, stream));
     else
@@ -261,9 +265,13 @@ extern "C" int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, con
       const int fs = l.shared_ff, E = l.experts, top = l.top, ff = l.ff, Z = M * top;
       MN_TRY(norm_stage(l.norm2, l.canon2, st->canon[ri] ? st->canon[ri] + canon_half : nullptr, &h, &h16));
       MN_TRY(linear(arith, M, h, W, h16, W, l.w_ff_in, d.n_ff_in, W, l.b_ff_in, fin, d.n_ff_in, gws, gwb, stream));
-      MN_TRY(mn_router_topk_rows(fin + 2 * fs, d.n_ff_in, M, E, top, tidx, tw, stream));
+      if (fs > 0 && !sah) {          // few rows (no bf16 copy wanted): the router's pick and the shared activation in one launch
+        MN_TRY(mn_router_topk_silu_rows(fin + 2 * fs, d.n_ff_in, M, E, top, tidx, tw, fin, d.n_ff_in, sa, fs, fs, stream));
+      } else {
+        MN_TRY(mn_router_topk_rows(fin + 2 * fs, d.n_ff_in, M, E, top, tidx, tw, stream));
+        if (fs > 0) MN_TRY(mn_silu_mul_rows(fin, d.n_ff_in, sa, fs, sah, fs, M, fs, stream));
+      }
       if (fs > 0) {
-        MN_TRY(mn_silu_mul_rows(fin, d.n_ff_in, sa, fs, sah, fs, M, fs, stream));
         MN_TRY(linear(arith, M, sa, fs, sah, fs, l.w_shared_down, W, fs, nullptr, sh, W, gws, gwb, stream));
       }
       const int32_t* so = nullptr;

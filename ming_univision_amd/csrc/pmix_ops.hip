@@ -162,6 +162,8 @@ struct RopeArgs {
   // decode rows only (ROW): the channel filter in front with its state, and the block means behind
   const bf16_t* w_conv; int conv; float* conv_state;
   float* pk; float* pv; int n_pool_max, pool;
+  // ... and the minGRU of the same rows, in extra workgroups of the launch (gru_n 0: none)
+  const float* zx; int64_t ldzx; const float* gg; int64_t ldgg; float* gru_state; int gru_n; float gru_scale; float* gru_out; int64_t ldgo;
 };
 
 // ROW: every row is alone in its sequence (a decode step).  The kernel then reads its channels through the short causal filter
@@ -172,6 +174,19 @@ template <bool ROW>
 __global__ __launch_bounds__(256) void rope_unit_append_kernel(RopeArgs a, int M) {
   const int hv = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, m = blockIdx.y;
   const int nh = a.H + 2 * a.G;
+  if (ROW && a.gru_n > 0 && (int)blockIdx.x >= (nh + 3) / 4) {      // the recurrence of this row: one thread per channel
+    const int c = ((int)blockIdx.x - (nh + 3) / 4) * 256 + threadIdx.x;
+    if (c >= a.gru_n) return;
+    float* sp = a.gru_state + (int64_t)a.row_seq[m] * a.gru_n + c;
+    const float S0 = a.row_slot[m] == 0 ? 0.f : *sp;
+    const float z = sigmoid_f(a.zx[(int64_t)m * a.ldzx + c]);
+    const float u = a.zx[(int64_t)m * a.ldzx + a.gru_n + c];
+    const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+    const float S = (1.0f - z) * S0 + z * cand;
+    a.gru_out[(int64_t)m * a.ldgo + c] = a.gru_scale * S * silu_f(a.gg[(int64_t)m * a.ldgg + c]);
+    *sp = S;
+    return;
+  }
   if (hv >= nh) return;
   const float* row = a.qkv + (int64_t)m * a.ldqkv;
   const int seq = a.row_seq[m], slot = a.row_slot[m];
@@ -866,7 +881,14 @@ __global__ __launch_bounds__(256) void mingru_pass3_kernel(MinGruArgs a) {
 // one wave per row: `top` rounds of arg-max (ties: the lower index), then the softmax over the chosen logits.  Lane l owns the
 // logits l, l + 64, ... and a bit per owned logit that says it has been chosen (E <= 4096).
 __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int64_t ld, int M, int E, int top,
-                                                          int32_t* __restrict__ idx, float* __restrict__ w) {
+                                                          int32_t* __restrict__ idx, float* __restrict__ w, const float* __restrict__ sx,
+                                                          int64_t ldsx, float* __restrict__ sy, int64_t ldsy, int sn) {
+  const int nb = (M + 3) / 4;
+  if ((int)blockIdx.x >= nb) {                          // extra workgroups: sy[m, c] = silu(sx[m, c]) * sx[m, sn + c]
+    const int per_row = (sn + 255) / 256, e = (int)blockIdx.x - nb, m = e / per_row, c = (e % per_row) * 256 + threadIdx.x;
+    if (c < sn) sy[(int64_t)m * ldsy + c] = silu_f(sx[(int64_t)m * ldsx + c]) * sx[(int64_t)m * ldsx + sn + c];
+    return;
+  }
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= M) return;
   const float* z = logits + (int64_t)row * ld;
@@ -989,7 +1011,7 @@ extern "C" int mn_rope_unit_append(const float* qkv, int64_t ldqkv, int M, int H
   MN_CHECK_ARG(dim >= 1 && dim <= 512 && vdim >= 1 && rot_dims >= 0 && rot_dims <= dim && (rot_dims % 2) == 0 && (rot_dims == 0 || freq),
                "mn_rope_unit_append: dim=%d (at most 512), rot_dims=%d (even, at most dim)", dim, rot_dims);
   RopeArgs a{qkv, ldqkv, H, G, dim, vdim, rot_dims, freq, mag, unit, eps, q_scale, row_seq, row_slot, q_out, ldq, k_arena, v_arena, t_max,
-             nullptr, 0, nullptr, nullptr, nullptr, 0, 0};
+             nullptr, 0, nullptr, nullptr, nullptr, 0, 0, nullptr, 0, nullptr, 0, nullptr, 0, 0.f, nullptr, 0};
   hipLaunchKernelGGL((rope_unit_append_kernel<false>), dim3((unsigned)mn_cdiv(H + 2 * G, 4), (unsigned)M), dim3(256), 0, mn_stream(stream), a, M);
   MN_CHECK_LAUNCH("mn_rope_unit_append");
   return MN_OK;
@@ -998,7 +1020,10 @@ extern "C" int mn_rope_unit_append(const float* qkv, int64_t ldqkv, int M, int H
 extern "C" int mn_filter_rope_append_rows(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, const uint16_t* w_conv, int conv,
                                           float* conv_state, int rot_dims, const float* freq, float mag, int unit, float eps, float q_scale,
                                           const int32_t* row_seq, const int32_t* row_slot, float* q_out, int64_t ldq, float* k_arena,
-                                          float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool, void* stream) {
+                                          float* v_arena, int t_max, float* pk, float* pv, int n_pool_max, int pool, const float* zx,
+                                          int64_t ldzx, const float* g, int64_t ldg, float* gru_state, int gru_n, float gru_scale, float* gru_out,
+                                          int64_t ldgo, void* stream) {
+  MN_CHECK_ARG(gru_n == 0 || (gru_n > 0 && zx && g && gru_state && gru_out), "mn_filter_rope_append_rows: bad recurrence args");
   MN_CHECK_ARG(qkv && row_seq && row_slot && q_out && k_arena && v_arena && M >= 1 && M <= 65535 && H >= 1 && G >= 1 && t_max >= 1,
                "mn_filter_rope_append_rows: bad args");
   MN_CHECK_ARG(dim >= 1 && dim <= 512 && vdim >= 1 && rot_dims >= 0 && rot_dims <= dim && (rot_dims % 2) == 0 && (rot_dims == 0 || freq),
@@ -1006,8 +1031,9 @@ extern "C" int mn_filter_rope_append_rows(const float* qkv, int64_t ldqkv, int M
   MN_CHECK_ARG(conv >= 0 && (conv == 0 || w_conv) && (conv <= 1 || conv_state) && pool >= 0 && (pool == 0 || (pk && pv && n_pool_max >= 1)),
                "mn_filter_rope_append_rows: bad filter or block arenas");
   RopeArgs a{qkv, ldqkv, H, G, dim, vdim, rot_dims, freq, mag, unit, eps, q_scale, row_seq, row_slot, q_out, ldq, k_arena, v_arena, t_max,
-             w_conv, conv, conv_state, pk, pv, n_pool_max, pool};
-  hipLaunchKernelGGL((rope_unit_append_kernel<true>), dim3((unsigned)mn_cdiv(H + 2 * G, 4), (unsigned)M), dim3(256), 0, mn_stream(stream), a, M);
+             w_conv, conv, conv_state, pk, pv, n_pool_max, pool, zx, ldzx, g, ldg, gru_state, gru_n, gru_scale, gru_out, ldgo};
+  hipLaunchKernelGGL((rope_unit_append_kernel<true>), dim3((unsigned)(mn_cdiv(H + 2 * G, 4) + mn_cdiv(gru_n, 256)), (unsigned)M), dim3(256), 0,
+                     mn_stream(stream), a, M);
   MN_CHECK_LAUNCH("mn_filter_rope_append_rows");
   return MN_OK;
 }
@@ -1174,8 +1200,19 @@ extern "C" int mn_mingru_rows_scan(const float* zx, int64_t ldzx, const float* g
 
 extern "C" int mn_router_topk_rows(const float* logits, int64_t ld, int M, int E, int top, int32_t* idx, float* w, void* stream) {
   MN_CHECK_ARG(logits && idx && w && M >= 1 && E >= 1 && E <= 4096 && top >= 1 && top <= E, "mn_router_topk_rows: bad args (E=%d top=%d)", E, top);
-  hipLaunchKernelGGL(router_topk_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), logits, ld, M, E, top, idx, w);
+  hipLaunchKernelGGL(router_topk_kernel, dim3((unsigned)mn_cdiv(M, 4)), dim3(256), 0, mn_stream(stream), logits, ld, M, E, top, idx, w,
+                     (const float*)nullptr, (int64_t)0, (float*)nullptr, (int64_t)0, 0);
   MN_CHECK_LAUNCH("mn_router_topk_rows");
+  return MN_OK;
+}
+
+extern "C" int mn_router_topk_silu_rows(const float* logits, int64_t ld, int M, int E, int top, int32_t* idx, float* w, const float* x,
+                                        int64_t ldx, float* y, int64_t ldy, int n, void* stream) {
+  MN_CHECK_ARG(logits && idx && w && x && y && M >= 1 && E >= 1 && E <= 4096 && top >= 1 && top <= E && n >= 1 &&
+                   mn_cdiv(M, 4) + (int64_t)M * mn_cdiv(n, 256) <= 0x7fffffff, "mn_router_topk_silu_rows: bad args (E=%d top=%d)", E, top);
+  hipLaunchKernelGGL(router_topk_kernel, dim3((unsigned)(mn_cdiv(M, 4) + (int64_t)M * mn_cdiv(n, 256))), dim3(256), 0, mn_stream(stream), logits,
+                     ld, M, E, top, idx, w, x, ldx, y, ldy, n);
+  MN_CHECK_LAUNCH("mn_router_topk_silu_rows");
   return MN_OK;
 }
 

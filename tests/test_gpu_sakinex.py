@@ -240,6 +240,10 @@ def test_decode_rows_filter_rotation_append_and_block_means_in_one_launch(H, G, 
     a = {k: v.cuda() for k, v in init.items()}
     b = {k: v.cuda() for k, v in init.items()}
     qa, qb, tmp = torch.empty(M, H * dim, device="cuda"), torch.empty(M, H * dim, device="cuda"), torch.empty(M, C, device="cuda")
+    ng = 300
+    zx, gg = torch.randn(M, 2 * ng + 1, generator=g).cuda(), torch.randn(M, ng, generator=g).cuda()
+    gst = torch.randn(n_seq, ng, generator=g)
+    gst_a, gst_b, go_a, go_b = gst.cuda(), gst.cuda(), torch.zeros(M, ng + 3, device="cuda"), torch.zeros(M, ng + 3, device="cuda")
     src, ld = pin, C + 7
     if conv:
         check(L.mn_tap_conv_rows(ptr(pin), C + 7, ptr(w), conv, ptr(a["state"]), ptr(seq), ptr(slot), ptr(back), ptr(tmp), C, M, C, stream()))
@@ -252,7 +256,11 @@ def test_decode_rows_filter_rotation_append_and_block_means_in_one_launch(H, G, 
                                       stream()))
     check(L.mn_filter_rope_append_rows(ptr(pin), C + 7, M, H, G, dim, vdim, ptr(w) if conv else None, conv, ptr(b["state"]), dims, ptr(freq), mag, 1, 1e-6,
                                        0.3, ptr(seq), ptr(slot), ptr(qb), H * dim, ptr(b["ka"]), ptr(b["va"]), t_max, ptr(b["pk"]) if pool else None,
-                                       ptr(b["pv"]) if pool else None, npm, pool, stream()))
+                                       ptr(b["pv"]) if pool else None, npm, pool, ptr(zx), 2 * ng + 1, ptr(gg), ng, ptr(gst_b), ng, 0.4, ptr(go_b), ng + 3,
+                                       stream()))
+    check(L.mn_mingru_rows(ptr(zx), 2 * ng + 1, ptr(gg), ng, ptr(gst_a), ptr(seq), ptr(slot), ptr(back), 0.4, ptr(go_a), ng + 3, None, 0, M, ng,
+                           stream()))
+    assert err(go_b[:, :ng], go_a[:, :ng].cpu()) < 1e-6 and err(gst_b, gst_a.cpu()) < 1e-6      # the recurrence of the same rows rides the launch
     assert err(qb, qa.cpu()) < 1e-6
     for k in a:
         assert err(b[k], a[k].cpu()) < 1e-6, k
@@ -408,6 +416,13 @@ def test_router_and_expert_operators():
     y = torch.empty(M, n, device="cuda")
     check(L.mn_silu_mul_rows(ptr(D(x)), 2 * n, ptr(y), n, None, 0, M, n, stream()))
     assert err(y, torch.nn.functional.silu(x[:, :n].double()) * x[:, n:].double()) < 1e-6
+    for M2, n2 in ((1, 300), (5, 37), (3, 700)):                   # the router's pick and the shared activation of few rows in one launch
+        z, x2 = torch.randn(M2, 9, generator=g), torch.randn(M2, 2 * n2 + 2, generator=g)
+        val, idx = torch.topk(z[:, :7].double(), 3, dim=-1)
+        di, dw, y2 = torch.empty(M2, 3, dtype=torch.int32, device="cuda"), torch.empty(M2, 3, device="cuda"), torch.zeros(M2, n2 + 1, device="cuda")
+        check(L.mn_router_topk_silu_rows(ptr(D(z)), 9, M2, 7, 3, ptr(di), ptr(dw), ptr(D(x2)), 2 * n2 + 2, ptr(y2), n2 + 1, n2, stream()))
+        assert torch.equal(di.cpu().long(), idx) and err(dw, torch.softmax(val, -1)) < 1e-6
+        assert err(y2[:, :n2], torch.nn.functional.silu(x2[:, :n2].double()) * x2[:, n2:2 * n2].double()) < 1e-6 and float(y2[:, n2].abs().max()) == 0.0
     for K_ in (K, 64):                                              # scalar and 8-wide weight loads
         a, w = torch.randn(M, K_, generator=g), _bf(torch.randn(E, n, K_, generator=g))
         idx = torch.randint(0, E, (M * top,), generator=g).to(torch.int32)
