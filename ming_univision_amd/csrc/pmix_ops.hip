@@ -149,6 +149,91 @@ __global__ __launch_bounds__(256) void axpy_rms_filter_kernel(AxpyRmsFilterArgs 
   }
 }
 
+// The same with 16-byte accesses: a thread owns NV groups of four consecutive channels (rows of n % 4 == 0 values at 16-byte aligned
+// addresses, at most 4 taps): a row of 2 048 values is 16 loads per thread instead of 80.
+template <int NV>
+__global__ __launch_bounds__(256) void axpy_rms_filter_vec_kernel(AxpyRmsFilterArgs a) {
+  __shared__ float red[8];
+  constexpr int MT = 4;
+  const int row = blockIdx.x, tid = threadIdx.x, n = a.n, ng = n / 4;
+  const bool filter = a.taps_w != nullptr && a.taps >= 1;
+  const int seq = filter ? a.row_seq[row] : 0, slot = filter ? a.row_slot[row] : 0;
+  float* const st0 = (filter && a.taps > 1) ? a.state + (int64_t)seq * (a.taps - 1) * n : nullptr;
+  const float* sbase = st0 ? st0 : a.x + (int64_t)row * a.ldx;
+  const int64_t sstr = st0 ? n : 0;
+  const int ns = st0 ? a.taps - 1 : 1;
+  float4 xv[NV], sv[NV][MT - 1];
+  float wv[NV][4], tv[NV][4][MT];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int gi = tid + 256 * i, gg = gi < ng ? gi : 0, c0 = 4 * gg;
+    float4 t = *reinterpret_cast<const float4*>(a.x + (int64_t)row * a.ldx + c0);
+    if (a.y) {
+      const float4 yv = *reinterpret_cast<const float4*>(a.y + (int64_t)row * a.ldy + c0);
+      t.x += a.mult * yv.x; t.y += a.mult * yv.y; t.z += a.mult * yv.z; t.w += a.mult * yv.w;
+    }
+    xv[i] = gi < ng ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+    const uint2 wq = *reinterpret_cast<const uint2*>(a.w + c0);
+    wv[i][0] = bf16lo_to_f32(wq.x); wv[i][1] = bf16hi_to_f32(wq.x); wv[i][2] = bf16lo_to_f32(wq.y); wv[i][3] = bf16hi_to_f32(wq.y);
+#pragma unroll
+    for (int k = 1; k < MT; ++k) {
+      const float4 v = *reinterpret_cast<const float4*>(sbase + (int64_t)(min(k, ns) - 1) * sstr + c0);
+      sv[i][k - 1] = (st0 && k < a.taps) ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (filter && a.taps == 4 && (((uintptr_t)a.taps_w) & 15) == 0) {      // four channels x four taps: 32 contiguous bytes
+      const uint4* tp = reinterpret_cast<const uint4*>(a.taps_w + (int64_t)c0 * 4);
+      const uint4 ta = tp[0], tb = tp[1];
+      const uint32_t wd[8] = {ta.x, ta.y, ta.z, ta.w, tb.x, tb.y, tb.z, tb.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {                        // tv[.][k]: the tap on the input k positions back = weight 3 - k
+        tv[i][e][3] = bf16lo_to_f32(wd[2 * e]); tv[i][e][2] = bf16hi_to_f32(wd[2 * e]);
+        tv[i][e][1] = bf16lo_to_f32(wd[2 * e + 1]); tv[i][e][0] = bf16hi_to_f32(wd[2 * e + 1]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int k = 0; k < MT; ++k) {
+          const float v = filter ? bf16_to_f32(a.taps_w[(int64_t)(c0 + e) * a.taps + max(a.taps - 1 - k, 0)]) : 0.f;
+          tv[i][e][k] = k < a.taps ? v : 0.f;
+        }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) s += xv[i].x * xv[i].x + xv[i].y * xv[i].y + xv[i].z * xv[i].z + xv[i].w * xv[i].w;
+  const float r = 1.0f / sqrtf(block_sum(s, red) / (float)n + a.eps);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int gi = tid + 256 * i, c0 = 4 * gi;
+    if (gi >= ng) continue;
+    if (a.y) *reinterpret_cast<float4*>(a.x + (int64_t)row * a.ldx + c0) = xv[i];
+    const float xe[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+    float nv[4], hv[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      nv[e] = xe[e] * r * wv[i][e];
+      hv[e] = nv[e];
+      if (filter) {
+        hv[e] += tv[i][e][0] * nv[e];
+#pragma unroll
+        for (int k = 1; k < MT; ++k) {
+          const float4 q = sv[i][k - 1];
+          const float se = e == 0 ? q.x : (e == 1 ? q.y : (e == 2 ? q.z : q.w));
+          if (k < a.taps && slot - k >= 0) hv[e] += tv[i][e][k] * se;
+        }
+      }
+    }
+    if (st0) {
+#pragma unroll
+      for (int k = MT - 2; k >= 1; --k)
+        if (k < a.taps - 1) *reinterpret_cast<float4*>(st0 + (int64_t)k * n + c0) = sv[i][k - 1];
+      *reinterpret_cast<float4*>(st0 + c0) = make_float4(nv[0], nv[1], nv[2], nv[3]);
+    }
+    *reinterpret_cast<float4*>(a.h + (int64_t)row * a.ldh + c0) = make_float4(hv[0], hv[1], hv[2], hv[3]);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------------------------
 // One wave per (row, head vector): q heads 0 .. H - 1, k heads H .. H + G - 1, v heads after them.  A lane holds the pairs
 // (i, i + half) for i = lane, lane + 64, ... and the values past rot_dims: at most 8 of each (dim <= 512).
@@ -991,6 +1076,17 @@ extern "C" int mn_axpy_rms_filter_rows(float* x, int64_t ldx, const float* y, in
   AxpyRmsFilterArgs a{x, ldx, y, ldy, mult, w, eps, taps_w, taps_w ? taps : 0, state, row_seq, row_slot, h, ldh, n};
   const int vpt = (n + 255) / 256;
   hipStream_t st = mn_stream(stream);
+  const bool vec = (n % 4) == 0 && a.taps <= 4 && (ldx % 4) == 0 && (ldh % 4) == 0 && (!y || (ldy % 4) == 0) &&
+                   ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)h) | ((uintptr_t)state)) & 15) == 0 && (((uintptr_t)w) & 7) == 0;
+  if (vec) {
+    const int nvg = (n / 4 + 255) / 256;
+    if (nvg <= 1) hipLaunchKernelGGL((axpy_rms_filter_vec_kernel<1>), dim3((unsigned)M), dim3(256), 0, st, a);
+    else if (nvg <= 2) hipLaunchKernelGGL((axpy_rms_filter_vec_kernel<2>), dim3((unsigned)M), dim3(256), 0, st, a);
+    else if (nvg <= 4) hipLaunchKernelGGL((axpy_rms_filter_vec_kernel<4>), dim3((unsigned)M), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((axpy_rms_filter_vec_kernel<8>), dim3((unsigned)M), dim3(256), 0, st, a);
+    MN_CHECK_LAUNCH("mn_axpy_rms_filter_rows");
+    return MN_OK;
+  }
 #define MN_RB(V_)                                                                                                   \
   do {                                                                                                              \
     if (a.taps <= 4) hipLaunchKernelGGL((axpy_rms_filter_kernel<V_, 4>), dim3((unsigned)M), dim3(256), 0, st, a); \

@@ -135,7 +135,8 @@ def _drop_device_copies():
 def test_residual_norm_rows_and_fused_decode_rows():
     check, stream, L, ptr = _api()
     g = torch.Generator().manual_seed(0)
-    for M, n, taps, eps in ((1, 44, 3, 1e-5), (5, 256, 1, 1e-6), (9, 1000, 8, 1e-3), (3, 300, 2, 1e-6)):
+    for M, n, taps, eps in ((1, 44, 3, 1e-5), (5, 256, 1, 1e-6), (9, 1000, 8, 1e-3), (3, 300, 2, 1e-6), (2, 2048, 4, 1e-6), (4, 1028, 4, 1e-6),
+                            (2, 250, 4, 1e-6), (3, 64, 1, 1e-6), (2, 520, 6, 1e-6)):
         x, y = torch.randn(M, n, generator=g) * 2, torch.randn(M, n, generator=g)
         w, tw = _bf(1 + 0.2 * torch.randn(n, generator=g)), _bf(0.5 * torch.randn(n, taps, generator=g))
         state = torch.randn(4, max(taps - 1, 1), n, generator=g)
